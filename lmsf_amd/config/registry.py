@@ -68,6 +68,8 @@ def resolve_architecture(config_dict: Dict[str, Any]) -> Architecture:
     archs = config_dict.get("architectures")
     if isinstance(archs, (list, tuple)) and archs:
         return get_architecture(str(archs[0]))
+    if isinstance(config_dict.get("architecture"), str):      # some configurations name it in the singular
+        return get_architecture(config_dict["architecture"])
     mt = config_dict.get("model_type")
     if isinstance(mt, str):
         for a in _ARCHITECTURES.values():

@@ -25,6 +25,26 @@ int lmsf_paged_attention_decode_mfma(const void* q, long q_stride, void* out, lo
     const int* pos, int nh, int nkv, int d, int ps, float scale, int window, int chunk, int n_splits, float* scratch,
     int order, hipStream_t stream);
 
+// group_norm.hip
+int lmsf_group_norm(const void* branch, int branch_dtype, long branch_stride, const float* wb, float* residual,
+    float* hist, long hist_stride, int hist_index, const float* mix, const float* wn, void* out, int out_dtype,
+    long out_stride, const int* rows, int n_rows, int W, int groups, float eps_b, float eps_n, hipStream_t stream);
+
+// latent.hip
+int lmsf_latent_cache_write(const void* x, int dtype, long x_stride, const float* w, float eps, const int* positions,
+    const float* table, int rot, int max_pos, const int* slots, void* k_pages, void* v_pages, long num_pages,
+    int n_tokens, int R, int dr, int D, int ps, hipStream_t stream);
+int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_head, const void* W, void* y, long y_stride,
+    int y_head, const void* gate, long gate_stride, int n_tokens, int H, int O, int K, hipStream_t stream);
+int lmsf_rope_tail(const void* x, int dtype, long x_stride, int x_head, int x_at, void* y, long y_stride, int y_head,
+    int y_at, const int* positions, const float* table, int rot, int max_pos, int n_tokens, int H, int dr,
+    hipStream_t stream);
+
+// moe.hip
+int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd, const int* ids,
+    const int* table, int vocab, int top, int E, float weight, const void* base, long base_stride, void* act,
+    void* out, long out_stride, int n_tokens, int F, int W, hipStream_t stream);
+
 // blas.hip
 int lmsf_blas_init(long workspace_bytes);
 int lmsf_blas_ready();

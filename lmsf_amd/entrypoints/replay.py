@@ -90,8 +90,12 @@ def main(argv=None) -> int:
         shutil.copyfile(args.random, os.path.join(model_dir, "config.json"))
     _say("torch ready after %.0f s; loading kernels and %s" % (time.time() - t0, args.model or args.random))
     num_pages = args.num_gpu_blocks if args.num_gpu_blocks else pages_for(args.max_tokens, args.block_size)
+    # no request can grow beyond the pool, whatever length the configuration allows
+    from lmsf_amd.config import load_model_config
+    longest = min(load_model_config(model_dir)[1].max_position_embeddings, num_pages * args.block_size)
     core = load_engine_core(model_dir, dtype=args.dtype, block_size=args.block_size, num_pages=num_pages,
-                            max_num_seqs=64, device=args.device, load_format=load_format, seed=args.seed)
+                            max_model_len=longest, max_num_seqs=64, device=args.device, load_format=load_format,
+                            seed=args.seed)
     _say("model %s ready after %.0f s: %s, %d pages of %d tokens" % (
         core.arch.name, time.time() - t0, args.dtype, num_pages, args.block_size))
     executor = core.executor

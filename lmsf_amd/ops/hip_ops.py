@@ -566,6 +566,155 @@ class HipOps:
         events[turn].record()
         return out
 
+    # ------------------------------------------------------------------ norm in groups, latent attention, experts
+
+    def group_norm(self, x: Optional[torch.Tensor] = None, x_weight: Optional[torch.Tensor] = None,
+                   residual: Optional[torch.Tensor] = None, out_weight: Optional[torch.Tensor] = None, groups: int = 1,
+                   x_eps: float = 1e-5, out_eps: float = 1e-5, out_dtype: Optional[torch.dtype] = None,
+                   rows: Optional[torch.Tensor] = None, history: Optional[torch.Tensor] = None, index: int = 0,
+                   mix: Optional[torch.Tensor] = None, want_out: bool = True) -> Optional[torch.Tensor]:
+        """RMS norm in ``groups`` equal consecutive parts of a row, gn(v; w) = v / rms of v's part * w, around a
+        float32 stream; every operand is optional (csrc/group_norm.hip):
+
+            r = (residual[rows] if residual is given else 0) + (gn(x; x_weight) if x is given else 0)
+            residual <- r                                     (x and residual given, no rows)
+            history[index] <- r; r = sum_j<=index mix[j] history[j]; residual <- r        (history given)
+            returns gn(r; out_weight) (or r itself without out_weight) in out_dtype, unless want_out is False
+
+        ``x`` is [N, W] float32 or bfloat16 with unit column stride (a view of a wider buffer will do),
+        ``residual`` contiguous float32 [N, W], ``history`` contiguous float32 [L, N, W], the weights float32 [W]."""
+        self._dev(x, x_weight, residual, out_weight, rows, history, mix)
+        ref = x if x is not None else residual
+        if ref is None or ref.dim() != 2:
+            raise ValueError("group_norm needs x or a residual, [N, W]")
+        N, W = ref.shape
+        if x is not None:
+            if x.stride(1) != 1 or x_weight is None:
+                raise ValueError("group_norm: x needs unit column stride and its weight")
+        for w in (x_weight, out_weight, mix):
+            if w is not None and (w.dtype != torch.float32 or not w.is_contiguous()):
+                raise ValueError("group_norm: weights must be contiguous float32")
+        if x_weight is not None and x_weight.shape != (W,) or out_weight is not None and out_weight.shape != (W,):
+            raise ValueError("group_norm: weights must be [%d]" % W)
+        if residual is not None:
+            if residual.dtype != torch.float32 or not residual.is_contiguous() or residual.shape[1] != W:
+                raise ValueError("group_norm: the residual stream must be contiguous float32 [N, %d]" % W)
+            if rows is None and residual.shape[0] != N:
+                raise ValueError("group_norm: x and the residual differ in rows")
+        self._i32(rows, "rows")
+        n_out = N if rows is None else rows.numel()
+        if rows is not None and x is not None:
+            raise ValueError("group_norm: rows select from the residual only")
+        hist_stride = 0
+        if history is not None:
+            if history.dtype != torch.float32 or not history.is_contiguous() or tuple(history.shape[1:]) != (N, W) \
+                    or not (0 <= index < history.shape[0]) or mix is None or mix.numel() < index + 1 \
+                    or residual is None or rows is not None:
+                raise ValueError("group_norm: history must be float32 [L > index, %d, %d] with index + 1 weights" % (N, W))
+            hist_stride = history.stride(0)
+        out = None
+        if want_out:
+            out = torch.empty((n_out, W), dtype=out_dtype or ref.dtype, device=ref.device)
+        self._check(self.lib.lmsf_group_norm(
+            _ptr(x), _code(x.dtype) if x is not None else F32, x.stride(0) if x is not None else W, _ptr(x_weight),
+            _ptr(residual), _ptr(history), hist_stride, int(index), _ptr(mix), _ptr(out_weight), _ptr(out),
+            _code(out.dtype) if out is not None else F32, W, _ptr(rows), n_out, W, int(groups), float(x_eps),
+            float(out_eps), self._stream()))
+        return out
+
+    def latent_cache_write(self, x: torch.Tensor, weight: torch.Tensor, eps: float, rank: int, rot_width: int,
+                           positions: torch.Tensor, table: torch.Tensor, slots: torch.Tensor, k_pages: torch.Tensor,
+                           v_pages: torch.Tensor) -> None:
+        """Per token: c = rms_norm(x[:rank]) * weight, r = rotate(x[rank:rank + rot_width]) by the token's position
+        (``table`` float32 [max_pos, rot] = [cos | sin], the first ``rot`` entries of r in pairs (i, i + rot/2));
+        [c | r | zeros] goes to the token's slot of ``k_pages`` [pages, 1, page_size, D] and of ``v_pages``
+        [pages, 1, D, page_size]. A negative slot stores nothing."""
+        self._dev(x, weight, positions, table, slots, k_pages, v_pages)
+        N = x.shape[0]
+        if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < rank + rot_width:
+            raise ValueError("latent_cache_write: x must be [N, >= %d] with unit column stride" % (rank + rot_width))
+        if weight.dtype != torch.float32 or weight.shape != (rank,) or not weight.is_contiguous():
+            raise ValueError("latent_cache_write: weight must be contiguous float32 [%d]" % rank)
+        if table.dtype != torch.float32 or table.dim() != 2 or not table.is_contiguous() or table.shape[1] > rot_width \
+                or table.shape[1] % 2:
+            raise ValueError("latent_cache_write: bad rotary table")
+        self._i32(positions, "positions", N)
+        self._i32(slots, "slots", N)
+        if k_pages.dim() != 4 or k_pages.shape[1] != 1 or k_pages.shape[3] < rank + rot_width or k_pages.dtype != x.dtype \
+                or not k_pages.is_contiguous():
+            raise ValueError("latent_cache_write: k_pages must be contiguous [pages, 1, page_size, >= %d] of %s"
+                             % (rank + rot_width, x.dtype))
+        P, _, ps, D = k_pages.shape
+        if tuple(v_pages.shape) != (P, 1, D, ps) or v_pages.dtype != x.dtype or not v_pages.is_contiguous():
+            raise ValueError("latent_cache_write: v_pages must be contiguous [%d, 1, %d, %d] of %s" % (P, D, ps, x.dtype))
+        self._check(self.lib.lmsf_latent_cache_write(
+            _ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), float(eps), _ptr(positions), _ptr(table),
+            table.shape[1], table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), P, N, int(rank), int(rot_width),
+            D, ps, self._stream()))
+
+    def head_linear(self, x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int,
+                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """Per-head products: out[n, h * out_head + o] = sum_k weight[h, o, k] x[n, h * x_head + k], times
+        sigmoid(gate[n, h]) if a gate is given. ``weight`` contiguous [H, O, K]; x, out and gate are views with
+        unit column stride whose first column is head 0's first entry."""
+        self._dev(x, weight, out, gate)
+        H, O, K = weight.shape
+        N = x.shape[0]
+        if not weight.is_contiguous() or weight.dtype != x.dtype or out.dtype != x.dtype:
+            raise ValueError("head_linear: weight must be contiguous and of x's dtype, as the output")
+        if x.stride(1) != 1 or out.stride(1) != 1 or x.shape[1] < (H - 1) * x_head + K \
+                or out.shape[1] < (H - 1) * out_head + O or out.shape[0] != N:
+            raise ValueError("head_linear: operands too narrow for %d heads" % H)
+        if gate is not None and (gate.dtype != x.dtype or gate.stride(1) != 1 or gate.shape[1] < H or gate.shape[0] != N):
+            raise ValueError("head_linear: gate must be [N, >= %d] of x's dtype" % H)
+        self._check(self.lib.lmsf_head_linear(
+            _ptr(x), _code(x.dtype), x.stride(0), int(x_head), _ptr(weight), _ptr(out), out.stride(0), int(out_head),
+            _ptr(gate), gate.stride(0) if gate is not None else 0, N, H, O, K, self._stream()))
+        return out
+
+    def rope_tail(self, x: torch.Tensor, x_head: int, x_at: int, out: torch.Tensor, out_head: int, out_at: int,
+                  heads: int, width: int, positions: torch.Tensor, table: torch.Tensor) -> None:
+        """For every head h: out[n, h * out_head + out_at + e] = rotate(x[n, h * x_head + x_at + e]) for e < width
+        (the first ``rot`` = table.shape[1] of them in pairs (e, e + rot/2), the others as they are); the rest of
+        the head behind them in ``out`` is zeroed."""
+        self._dev(x, out, positions, table)
+        N = x.shape[0]
+        if x.stride(1) != 1 or out.stride(1) != 1 or x.shape[1] < heads * x_head or out.shape[1] < heads * out_head \
+                or out.shape[0] != N or out.dtype != x.dtype:
+            raise ValueError("rope_tail: operands too narrow for %d heads" % heads)
+        if table.dtype != torch.float32 or table.dim() != 2 or not table.is_contiguous() or table.shape[1] > width:
+            raise ValueError("rope_tail: bad rotary table")
+        self._i32(positions, "positions", N)
+        self._check(self.lib.lmsf_rope_tail(
+            _ptr(x), _code(x.dtype), x.stride(0), int(x_head), int(x_at), _ptr(out), out.stride(0), int(out_head),
+            int(out_at), _ptr(positions), _ptr(table), table.shape[1], table.shape[0], N, int(heads), int(width),
+            self._stream()))
+
+    def table_moe(self, h: torch.Tensor, w_gate_up: torch.Tensor, w_down: torch.Tensor, token_ids: torch.Tensor,
+                  table: torch.Tensor, weight: float, base: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out[n] = base[n] + weight * sum_k down_e(silu(gate_e h[n]) * up_e h[n]) over e = table[token_ids[n], k].
+        ``w_gate_up`` [E, 2 F, W] (gate rows first), ``w_down`` [E, W, F], ``table`` int32 [vocab, top]."""
+        self._dev(h, w_gate_up, w_down, token_ids, table, base)
+        N, W = h.shape
+        E, F2, _ = w_gate_up.shape
+        F = F2 // 2
+        if tuple(w_gate_up.shape) != (E, 2 * F, W) or tuple(w_down.shape) != (E, W, F) or not w_gate_up.is_contiguous() \
+                or not w_down.is_contiguous() or w_gate_up.dtype != h.dtype or w_down.dtype != h.dtype:
+            raise ValueError("table_moe: expert weights must be contiguous [E, 2F, W] and [E, W, F] of h's dtype")
+        if h.stride(1) != 1 or (base is not None and (base.shape != h.shape or base.stride(1) != 1 or base.dtype != h.dtype)):
+            raise ValueError("table_moe: h and base must be [N, W] with unit column stride")
+        self._i32(token_ids, "token_ids", N)
+        if table.dtype != torch.int32 or table.dim() != 2 or not table.is_contiguous():
+            raise ValueError("table_moe: table must be contiguous int32 [vocab, top]")
+        vocab, top = table.shape
+        act = torch.empty((N * top, F), dtype=h.dtype, device=h.device)
+        out = torch.empty((N, W), dtype=h.dtype, device=h.device)
+        self._check(self.lib.lmsf_table_moe(
+            _ptr(h), _code(h.dtype), h.stride(0), _ptr(w_gate_up), _ptr(w_down), _ptr(token_ids), _ptr(table), vocab,
+            top, E, float(weight), _ptr(base), base.stride(0) if base is not None else 0, _ptr(act), _ptr(out),
+            out.stride(0), N, F, W, self._stream()))
+        return out
+
     # ------------------------------------------------------------------ feed-forward
 
     def gated_act(self, gu: torch.Tensor, kind: str = "silu") -> torch.Tensor:

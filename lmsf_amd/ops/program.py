@@ -627,6 +627,10 @@ def record_program(model, hip_ops, in_python: Optional[Callable[[Any, str], bool
     if n_groups > MAX_GROUPS:
         last_failure = "%d cache groups, the step program takes %d" % (n_groups, MAX_GROUPS)
         return None
+    fixed = [type(p).__name__ for p in model.parts() if not getattr(p, "recordable", True)]
+    if fixed:
+        last_failure = "parts that run outside the step program: %s" % ", ".join(sorted(set(fixed)))
+        return None
     rec = Recorder(rt.dtype, model.spec.hidden_size, model.spec.vocab_size)
     rec.roles = {id(model.embedding): "embedding", id(model.head): "head"}
     rec.in_python = in_python

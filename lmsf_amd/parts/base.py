@@ -86,7 +86,8 @@ class TensorDecl:
     ``keeps_float32``: a tensor stored in 32 bits stays so in a bfloat16 run (the norms' weights: their kernels
     compute in float32 anyway and take the weight as it is); the matrices of the products are cast as the
     reference casts everything (core/src/model_executor/models/model_factory.rs:124-139). ``init`` says how
-    the random-weights mode fills it: "normal" (mean 0, the mode's standard deviation), "ones" or "zeros"."""
+    the random-weights mode fills it: "normal" (mean 0, the mode's standard deviation), "ones", "zeros", "last_one"
+    (zeros and a final 1) or, for an integer table, "choices:E" (every row distinct numbers below E)."""
 
     shape: Tuple[int, ...]
     kind: str = "float"
@@ -142,6 +143,11 @@ class Part:
     model says so; a part that loops over the step's requests in Python leaves it False."""
 
     graph_safe = False
+
+    # False: the part's kernel calls are not among the operations of the recorded step program and it does not run
+    # as one of its callbacks either; a model with such a part runs part by part (captured as a graph all the same
+    # where every part is ``graph_safe``).
+    recordable = True
 
     # A mixer or feed-forward whose ``forward`` takes ``pending_ok=True`` and may then return its last
     # product unfinished (ops.handles.PendingProduct) sets this; a norm that takes such a branch in

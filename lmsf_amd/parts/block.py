@@ -3,7 +3,7 @@ from typing import Optional
 
 import torch
 
-from .base import Block, CacheBinding, register_part
+from .base import Block, CacheBinding, Runtime, build_part, register_part
 
 
 @register_part("block", "prenorm_residual")
@@ -44,3 +44,67 @@ class PreNormResidualBlock(Block):
         if self.feed_forward.may_return_pending and self.pending_output_ok:
             return self.feed_forward.forward(h, pending_ok=True)
         return self.feed_forward.forward(h)
+
+
+@register_part("block", "sandwich_depth_average")
+class SandwichDepthBlock(Block):
+    """A norm before and after each sublayer, and a weighted average over depth:
+
+        x += norm_b(mixer(norm_a(x)));   x += norm_d(ffn(norm_c(x)));   X_k = x;   x = sum_j<=k mix[j] X_j
+
+    with X_0 the embedding's output and X_k the result of the k-th layer run (k = ``depth``), before the
+    averaging. The stream and every X_j are float32. The results lie in one buffer [depth_total + 1, N, W] that
+    the first block of a step allocates and the others find in ``ctx.aux``. The addition after the mixer and the
+    norm before the feed-forward are one kernel; so are the addition after the feed-forward, the storing of
+    X_k and the averaging. Nothing is left to add when the block returns.
+
+    The reference's only arrangement is the pre-norm one above (core/src/model_executor/models/llama/llama.rs:286-340).
+    """
+
+    graph_safe = True
+    recordable = False
+
+    ROLES = ("pre_mixer", "post_mixer")          # "pre_ffn" and "post_ffn" too where there is a feed-forward
+
+    def __init__(self, prefix: str, rt: Runtime, mixer, feed_forward, norms, depth: int, depth_total: int,
+                 mix=None):
+        super().__init__(prefix, rt, mixer, feed_forward, norms)
+        self.depth, self.depth_total = int(depth), int(depth_total)
+        if not (1 <= self.depth <= self.depth_total):
+            raise ValueError("block %s: depth %d of %d" % (prefix, self.depth, self.depth_total))
+        self.has_ffn = not getattr(feed_forward, "absent", False)
+        if self.has_ffn and not ("pre_ffn" in norms and "post_ffn" in norms):
+            raise ValueError("block %s needs the norms pre_ffn and post_ffn around its feed-forward" % prefix)
+        self.mix = build_part("norm", mix, prefix, rt) if mix is not None else None
+        self._ffn_takes_ids = bool(getattr(feed_forward, "needs_token_ids", False))
+
+    def children(self):
+        return super().children() + ([self.mix] if self.mix is not None else [])
+
+    def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx, binding: CacheBinding):
+        if branch is not None:
+            raise ValueError("sandwich_depth_average takes no branch that is still to be added")
+        n = self.norms
+        hist = ctx.aux.get("depth_history")
+        if self.depth == 1 or hist is None or hist.shape[1:] != residual.shape:
+            hist = torch.empty((self.depth_total + 1,) + tuple(residual.shape), dtype=torch.float32,
+                               device=residual.device)
+            hist[0].copy_(residual)
+            ctx.aux["depth_history"] = hist
+        mix = self.mix.weight if self.mix is not None else None
+        h = n["pre_mixer"].forward(residual)
+        a = self.mixer.forward(h, ctx, binding)
+        if not self.has_ffn:
+            self._close(n["post_mixer"], a, residual, hist, mix)
+            return None
+        h = n["post_mixer"].add_normed(a, residual, then=n["pre_ffn"])
+        f = self.feed_forward.forward(h, token_ids=ctx.token_ids) if self._ffn_takes_ids else self.feed_forward.forward(h)
+        self._close(n["post_ffn"], f, residual, hist, mix)
+        return None
+
+    def _close(self, norm, branch, residual, hist, mix) -> None:
+        if mix is None:
+            norm.add_normed(branch, residual)
+            hist[self.depth].copy_(residual)
+        else:
+            norm.add_normed(branch, residual, history=hist, index=self.depth, mix=mix)

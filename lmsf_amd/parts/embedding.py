@@ -21,7 +21,8 @@ class TokenEmbedding(Part):
                  weight_name: str = "weight"):
         super().__init__(prefix, rt)
         self.vocab_size, self.hidden_size, self.scale = int(vocab_size), int(hidden_size), float(scale)
-        self.weight_name = "%s.%s" % (prefix, weight_name)
+        # (weight_name "": the table is the tensor ``prefix`` itself)
+        self.weight_name = "%s.%s" % (prefix, weight_name) if weight_name else prefix
         self.weight: Optional[torch.Tensor] = None
 
     def checkpoint_tensors(self) -> Dict[str, TensorDecl]:

@@ -16,13 +16,15 @@ class FusedLinear(Part):
     """One matrix product whose weight rows are the concatenation of several checkpoint tensors.
 
     ``sources`` is a list of (checkpoint sub-name, rows): the tensor ``prefix.sub-name.weight`` has
-    shape [rows, in_features] and, with ``bias``, ``prefix.sub-name.bias`` has [rows]."""
+    shape [rows, in_features] and, with ``bias``, ``prefix.sub-name.bias`` has [rows]. With ``bare_names`` the
+    matrix is the tensor ``prefix.sub-name`` itself (checkpoints that name a matrix without ".weight")."""
 
     graph_safe = True
 
     def __init__(self, prefix: str, rt: Runtime, in_features: int, sources: Sequence[Tuple[str, int]],
-                 bias: bool = False):
+                 bias: bool = False, bare_names: bool = False):
         super().__init__(prefix, rt)
+        self.bare_names = bool(bare_names)
         if not sources:
             raise ValueError("FusedLinear needs at least one source")
         self.in_features = int(in_features)
@@ -33,6 +35,8 @@ class FusedLinear(Part):
         self.bias: Optional[torch.Tensor] = None
 
     def _name(self, sub: str, what: str) -> str:
+        if self.bare_names and what == "weight":
+            return "%s.%s" % (self.prefix, sub) if self.prefix else sub
         return "%s.%s.%s" % (self.prefix, sub, what) if self.prefix else "%s.%s" % (sub, what)
 
     def checkpoint_tensors(self) -> Dict[str, TensorDecl]:
@@ -89,5 +93,6 @@ class FusedLinear(Part):
 class Linear(FusedLinear):
     """A single checkpoint matrix ``prefix.name.weight`` [out_features, in_features]."""
 
-    def __init__(self, prefix: str, rt: Runtime, name: str, in_features: int, out_features: int, bias: bool = False):
-        super().__init__(prefix, rt, in_features, [(name, out_features)], bias)
+    def __init__(self, prefix: str, rt: Runtime, name: str, in_features: int, out_features: int, bias: bool = False,
+                 bare_names: bool = False):
+        super().__init__(prefix, rt, in_features, [(name, out_features)], bias, bare_names)

@@ -15,14 +15,15 @@ class GatedMLP(FeedForward):
 
     def __init__(self, prefix: str, rt: Runtime, hidden_size: int, intermediate_size: int, activation: str = "silu",
                  bias: bool = False, gate_name: str = "gate_proj", up_name: str = "up_proj",
-                 down_name: str = "down_proj"):
+                 down_name: str = "down_proj", bare_names: bool = False):
         super().__init__(prefix, rt)
         if activation not in ("silu", "gelu"):
             raise ValueError("gated_mlp activation %r unknown (silu, gelu)" % activation)
         self.activation = activation
         self.gate_up = FusedLinear(prefix, rt, hidden_size,
-                                   [(gate_name, intermediate_size), (up_name, intermediate_size)], bias=bias)
-        self.down = Linear(prefix, rt, down_name, intermediate_size, hidden_size, bias=bias)
+                                   [(gate_name, intermediate_size), (up_name, intermediate_size)], bias=bias,
+                                   bare_names=bare_names)
+        self.down = Linear(prefix, rt, down_name, intermediate_size, hidden_size, bias=bias, bare_names=bare_names)
 
     def children(self):
         return [self.gate_up, self.down]

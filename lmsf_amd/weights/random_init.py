@@ -3,7 +3,8 @@
 The reference has no such mode (candle ``Init`` hints exist only as call arguments,
 tops/src/rms_norm.rs:42-46). Values are drawn per tensor from a generator seeded by
 (seed, tensor name), so they do not depend on the order in which tensors are made:
-matrices and biases N(0, std), norm weights 1.
+matrices and biases N(0, std), norm weights 1, integer tables 0 unless their part makes them
+(``TensorDecl.init`` "choices:E": every row distinct numbers below E).
 """
 import hashlib
 import json
@@ -32,11 +33,23 @@ def random_tensor(name: str, decl: TensorDecl, seed: int, std: float, dtype: tor
     """The tensor ``name`` of the random model ``seed``. Values are made in float32 on ``device``
     and rounded to ``dtype``; CPU and GPU generators differ, a model is tied to where it was made."""
     if decl.kind == "int":
+        if decl.init.startswith("choices:"):
+            # every row: distinct numbers below the bound named after the colon
+            bound = int(decl.init.split(":")[1])
+            gen = torch.Generator(device="cpu")
+            gen.manual_seed(tensor_seed(seed, name))
+            rows = [torch.randperm(bound, generator=gen)[:decl.shape[1]] for _ in range(decl.shape[0])]
+            return torch.stack(rows).to(torch.int32).to(device)
         return torch.zeros(decl.shape, dtype=torch.int32, device=device)
     if decl.init == "ones":
         return torch.ones(decl.shape, dtype=dtype, device=device)
     if decl.init == "zeros":
         return torch.zeros(decl.shape, dtype=dtype, device=device)
+    if decl.init == "last_one":
+        # weights of an average that passes its last term on unchanged
+        t = torch.zeros(decl.shape, dtype=dtype, device=device)
+        t.reshape(-1)[-1] = 1
+        return t
     if decl.init != "normal":
         raise ValueError("tensor %r: unknown init %r" % (name, decl.init))
     gen = torch.Generator(device=device)

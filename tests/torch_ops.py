@@ -144,6 +144,84 @@ class TorchOps:
             out[t] = torch.einsum("hn,nhd->hd", pr, vals).reshape(nh * d).to(q.dtype)
         return out
 
+    # ------------------------------------------------------------ norm in groups, latent attention, experts
+    @staticmethod
+    def _gn(v, w, groups, eps):
+        n, W = v.shape
+        p = v.reshape(n, groups, W // groups)
+        return (p / torch.sqrt((p * p).mean(dim=-1, keepdim=True) + eps)).reshape(n, W) * w
+
+    def group_norm(self, x=None, x_weight=None, residual=None, out_weight=None, groups=1, x_eps=1e-5, out_eps=1e-5,
+                   out_dtype=None, rows=None, history=None, index=0, mix=None, want_out=True):
+        ref = x if x is not None else residual
+        r = None
+        if x is not None:
+            r = self._gn(x.to(torch.float32), x_weight, groups, x_eps)
+        if residual is not None:
+            base = residual if rows is None else residual[rows.long()]
+            r = base if r is None else base + r
+            if x is not None and rows is None and history is None:
+                residual.copy_(r)
+        if history is not None:
+            history[index].copy_(r)
+            r = sum(mix[j] * history[j] for j in range(index + 1))
+            residual.copy_(r)
+        if not want_out:
+            return None
+        if out_weight is not None:
+            r = self._gn(r, out_weight, groups, out_eps)
+        return r.to(out_dtype or ref.dtype)
+
+    @staticmethod
+    def _rotate(v, cs, rot):
+        half = rot // 2
+        c, s = cs[..., :half], cs[..., half:rot]
+        a, b = v[..., :half], v[..., half:rot]
+        return torch.cat([a * c - b * s, b * c + a * s, v[..., rot:]], dim=-1)
+
+    def latent_cache_write(self, x, weight, eps, rank, rot_width, positions, table, slots, k_pages, v_pages):
+        ps, D = k_pages.shape[2], k_pages.shape[3]
+        xf = x.to(torch.float32)
+        c = self._gn(xf[:, :rank], weight, 1, eps)
+        r = self._rotate(xf[:, rank:rank + rot_width], table[positions.long()], table.shape[1])
+        row = torch.zeros((x.shape[0], D), dtype=torch.float32)
+        row[:, :rank], row[:, rank:rank + rot_width] = c, r
+        row = row.to(k_pages.dtype)
+        for n in range(x.shape[0]):
+            s = int(slots[n])
+            if s >= 0:
+                k_pages[s // ps, 0, s % ps, :] = row[n]
+                v_pages[s // ps, 0, :, s % ps] = row[n]
+
+    def head_linear(self, x, x_head, weight, out, out_head, gate=None):
+        H, O, K = weight.shape
+        for h in range(H):
+            y = x[:, h * x_head:h * x_head + K].to(torch.float32) @ weight[h].to(torch.float32).t()
+            if gate is not None:
+                y = y * torch.sigmoid(gate[:, h:h + 1].to(torch.float32))
+            out[:, h * out_head:h * out_head + O] = y.to(out.dtype)
+        return out
+
+    def rope_tail(self, x, x_head, x_at, out, out_head, out_at, heads, width, positions, table):
+        cs = table[positions.long()]
+        for h in range(heads):
+            v = x[:, h * x_head + x_at:h * x_head + x_at + width].to(torch.float32)
+            out[:, h * out_head + out_at:h * out_head + out_at + width] = self._rotate(v, cs, table.shape[1]).to(out.dtype)
+            out[:, h * out_head + out_at + width:(h + 1) * out_head] = 0
+
+    def table_moe(self, h, w_gate_up, w_down, token_ids, table, weight, base=None):
+        F = w_gate_up.shape[1] // 2
+        out = torch.zeros(h.shape, dtype=torch.float32)
+        for n in range(h.shape[0]):
+            for e in table[int(token_ids[n])].tolist():
+                gu = (w_gate_up[e].to(torch.float32) @ h[n].to(torch.float32)).to(h.dtype).to(torch.float32)
+                a = (gu[:F] / (1.0 + torch.exp(-gu[:F])) * gu[F:]).to(h.dtype).to(torch.float32)
+                out[n] += w_down[e].to(torch.float32) @ a
+        out = out * weight
+        if base is not None:
+            out = out + base.to(torch.float32)
+        return out.to(h.dtype)
+
     # ------------------------------------------------------------ feed-forward / linear
     def gated_act(self, gu, kind="silu"):
         I = gu.shape[1] // 2

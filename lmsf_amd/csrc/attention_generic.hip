@@ -1,5 +1,5 @@
 // Paged attention, general form: any number of query tokens per request, any head size that is a
-// multiple of 4 up to 256, any page size, float32 or bfloat16 storage, float32 arithmetic.
+// multiple of 4 up to 1024, any page size, float32 or bfloat16 storage, float32 arithmetic.
 //
 // Query token t belongs to request segment seg[t] and stands at position pos[t]. It attends to
 // the keys at positions j in [max(0, pos - window + 1), pos] of that request, read from the pages
@@ -16,7 +16,8 @@
 //
 // One workgroup of 256 threads per (token, head): keys are taken 256 at a time, one key per
 // thread for the scores, an online softmax across chunks, and the P V product with the threads
-// arranged as (key group, output dim).
+// arranged as (key group, output dim); a head wider than 256 has one key group and up to four output
+// dims a thread.
 #include "common.h"
 
 #include <math.h>
@@ -44,10 +45,11 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
 
   for (int i = tid; i < d; i += GEN_THREADS) sq[i] = to_f32<T>(q[(long)t * q_stride + h * d + i]) * scale;
 
-  const int ngroups = GEN_THREADS / d > 0 ? GEN_THREADS / d : 1;  // d <= 256
+  const int ngroups = GEN_THREADS / d > 0 ? GEN_THREADS / d : 1;
   const int og = tid / d, oi = tid % d;                            // (key group, output dim) of this thread
   const bool pv_active = og < ngroups;
   float acc = 0.f, m = -INFINITY, l = 0.f;
+  float wide[3] = {0.f, 0.f, 0.f};                                 // output dims tid + 256, + 512, + 768 (d > 256)
   __syncthreads();
 
   for (int j0 = lo; j0 <= p; j0 += GEN_THREADS) {
@@ -73,6 +75,9 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
     const float corr = (m == -INFINITY) ? 0.f : expf(m - m_new);
     l = l * corr + csum;
     acc *= corr;
+    if (d > GEN_THREADS) {
+      wide[0] *= corr; wide[1] *= corr; wide[2] *= corr;
+    }
     m = m_new;
     __syncthreads();
     if (pv_active) {
@@ -80,6 +85,13 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
       for (int jj = og; jj < n; jj += ngroups) {
         const int row = srow[jj], head_base = row / ps, off = row - head_base * ps;
         acc += sp[jj] * to_f32<T>(v_pages[((long)head_base * d + oi) * ps + off]);
+        if (d > GEN_THREADS) {
+#pragma unroll
+          for (int r = 0; r < 3; ++r) {
+            const int o2 = tid + (r + 1) * GEN_THREADS;
+            if (o2 < d) wide[r] += sp[jj] * to_f32<T>(v_pages[((long)head_base * d + o2) * ps + off]);
+          }
+        }
       }
     }
     __syncthreads();
@@ -91,6 +103,13 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
     for (int gg = 0; gg < ngroups; ++gg) o += sacc[gg * d + tid];
     out[(long)t * out_stride + h * d + tid] = from_f32<T>(o / l);
   }
+  if (d > GEN_THREADS) {
+#pragma unroll
+    for (int r = 0; r < 3; ++r) {
+      const int o2 = tid + (r + 1) * GEN_THREADS;
+      if (o2 < d) out[(long)t * out_stride + h * d + o2] = from_f32<T>(wide[r] / l);
+    }
+  }
 }
 
 extern "C" int lmsf_paged_attention_generic(const void* q, long q_stride, void* out, long out_stride,
@@ -101,7 +120,7 @@ extern "C" int lmsf_paged_attention_generic(const void* q, long q_stride, void* 
   LMSF_CHECK(q && out && k_pages && v_pages && block_tables && seg && pos, "paged_attention: null pointer");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "paged_attention: unknown dtype code %d", dtype);
   LMSF_CHECK(nh > 0 && nkv > 0 && nh % nkv == 0, "paged_attention: heads %d not a multiple of kv heads %d", nh, nkv);
-  LMSF_CHECK(d > 0 && d % 4 == 0 && d <= 256, "paged_attention: head size %d not supported (multiple of 4, <= 256)", d);
+  LMSF_CHECK(d > 0 && d % 4 == 0 && d <= 1024, "paged_attention: head size %d not supported (multiple of 4, <= 1024)", d);
   LMSF_CHECK(ps > 0 && bt_width > 0 && num_pages > 0, "paged_attention: bad page geometry");
   LMSF_CHECK(num_pages * nkv * ps < 2147483647L, "paged_attention: cache too large for 32-bit row indices");
   LMSF_CHECK(q_stride >= (long)nh * d && out_stride >= (long)nh * d, "paged_attention: row strides too small");

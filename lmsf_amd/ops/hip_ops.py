@@ -424,13 +424,14 @@ class HipOps:
     # ------------------------------------------------------------------ attention
 
     @staticmethod
-    def check_head_dim(d: int) -> None:
+    def check_head_dim(d: int, limit: int = 256) -> None:
         """Raises if no attention kernel takes head size ``d``: the matrix-core kernels take multiples of 16
-        up to 256 (bfloat16), the general kernel multiples of 4 up to 256 (either dtype). Parts ask this when
-        they are built, before any weight is loaded."""
-        if d <= 0 or d % 4 != 0 or d > 256:
+        up to 256 (bfloat16), the general kernel multiples of 4 up to 1,024 (either dtype). Parts ask this when
+        they are built, before any weight is loaded; ``limit`` is the widest head the part wants served (256
+        keeps a part on kernels that have a matrix-core form)."""
+        if d <= 0 or d % 4 != 0 or d > min(limit, 1024):
             raise ValueError("head size %d is not supported by the attention kernels: they take multiples of 4 "
-                             "up to 256 (multiples of 16 on the matrix cores)" % d)
+                             "up to %d (multiples of 16 up to 256 on the matrix cores)" % (d, min(limit, 1024)))
 
     def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                         block_tables: torch.Tensor, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, d: int,

@@ -206,7 +206,7 @@ class Recorder:
             setattr(op, k, v)
         self.ops.append(op)
 
-    def check_head_dim(self, d: int) -> None:      # parts are already built; nothing to ask
+    def check_head_dim(self, d: int, limit: int = 256) -> None:      # parts are already built; nothing to ask
         pass
 
     # -- the kernels' methods

@@ -61,7 +61,7 @@ class LatentAttention(Mixer):
         self.D = (self.R + self.dr + 15) // 16 * 16
         check = getattr(rt.ops, "check_head_dim", None)
         if check is not None:
-            check(self.D)
+            check(self.D, 1024)      # beyond 256 the general attention kernel serves it
         nm = dict(dq="dq", dkv="dkv", g="g", uq="uq", uk="uk", uv="uv", o="o", dq_norm="dq.norm", dkv_norm="dkv.norm")
         nm.update(names or {})
         # one product for everything that reads the layer's input: query latent, (key/value latent,) gates

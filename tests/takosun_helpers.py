@@ -34,7 +34,8 @@ def layer(m, mlp):
 
 
 # P: two heads, values wider than keys, two experts of three per token, a borrowed latent two layers back, one
-# norm group; Q: five heads, sizes that are no powers of two, a layer without feed-forward, experts without a
+# norm group; S: sizes that are multiples of 4 at most, with a latent wider than the matrix-core attention's heads;
+# Q: five heads, sizes that are no powers of two, a layer without feed-forward, experts without a
 # shared one, four norm groups; R: one head, a single expert per token, three layers on one latent.
 CONFIGS = {
     "P": {"architecture": "Takosun", "vocab": 97, "width": 64, "norm": {"eps": 1e-5, "groups": 1}, "layers": [
@@ -47,6 +48,10 @@ CONFIGS = {
         layer(mixer(5, 24, 16, 8, 40, 56, base=50000.0, kv_from=0, scale=0.3), moe(24, 5, 1)),
         layer(mixer(3, 8, 32, 40, 24, 16), dense(72)),
         layer(mixer(3, 8, 32, 40, 24, 16, kv_from=2), dense(200)),
+    ]},
+    "S": {"architecture": "Takosun", "vocab": 61, "width": 36, "norm": {"eps": 1e-5, "groups": 3}, "layers": [
+        layer(mixer(3, 12, 20, 6, 300, 20), moe(10, 3, 2, shared=50)),
+        layer(mixer(2, 4, 20, 28, 300, 44, kv_from=0), dense(52)),
     ]},
     "R": {"architecture": "Takosun", "vocab": 50, "width": 32, "norm": {"eps": 1e-5, "groups": 2}, "layers": [
         layer(mixer(1, 32, 4, 16, 12, 8), moe(16, 2, 1, shared=8)),

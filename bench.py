@@ -405,6 +405,65 @@ def further_shape_points(args, points, peak):
         points["llama70b_error"] = err
 
 
+def takosun_shapes(name):
+    """A Takosun configuration at sizes that resemble a real model's layers, and the Llama configuration of equal
+    width, depth, heads and feed-forward size (dense layers) beside it. Every second layer reads the latent of the
+    layer before it and has experts instead of a dense feed-forward."""
+    sizes = {
+        # width, layers, heads, unrotated / rotated / value size of a head, latent, query latent, dense ff,
+        # experts, their ff, experts a token, shared ff, vocabulary
+        "2b": (2048, 8, 16, 64, 32, 64, 224, 768, 8192, 16, 1024, 2, 2048, 32000),
+        "7b": (4096, 8, 32, 96, 32, 128, 224, 1536, 14336, 32, 2048, 2, 4096, 32000),
+    }[name]
+    W, L, H, dn, dr, dv, R, Q, ff, E, eff, top, sff, V = sizes
+    layers = []
+    for i in range(L):
+        m = {"heads": H, "dim": dn, "rot_dim": dr, "vdim": dv, "kv_rank": R, "q_rank": Q,
+             "rot": {"base": 10000.0, "dims": dr}, "scale": (dn + dr) ** -0.5}
+        if i % 2:
+            m["kv_from"] = i - 1
+            mlp = {"kind": "moe", "expert": {"ff": eff}, "router": {"experts": E, "top": top}, "shared": {"ff": sff}}
+        else:
+            mlp = {"kind": "dense", "ff": ff}
+        layers.append({"type": "latent_attention", "mixer": m, "mlp": mlp})
+    tako = {"architecture": "Takosun", "vocab": V, "width": W, "norm": {"eps": 1e-5, "groups": 2}, "layers": layers,
+            "max_position_embeddings": 8192, "torch_dtype": "bfloat16"}
+    llama = dict(LLAMA3_8B, vocab_size=V, hidden_size=W, intermediate_size=ff, num_hidden_layers=L,
+                 num_attention_heads=H, num_key_value_heads=max(1, H // 4), head_dim=dn + dr, bos_token_id=1,
+                 eos_token_id=2)
+    return tako, llama
+
+
+def takosun_run(args):
+    """``--workload takosun``: prefill and decode of a Takosun model beside the Llama model of equal size; one JSON
+    line. Decode: ``--steps`` steps at batch 1, 8 and 64 after 512-token prompts; prefill: one request of 512 and of
+    2,048 tokens."""
+    import gc
+    import torch
+    out = {"metric": "takosun_beside_llama", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+           "steps": args.steps, "warmup": args.warmup, "config": {"sizes": args.takosun_sizes}, "models": {}}
+    for name, cfg in zip(("takosun", "llama"), takosun_shapes(args.takosun_sizes)):
+        engine = make_engine(cfg, args, max_num_seqs=64, dtype=args.dtype)
+        m = {"weight_gb": round(weight_bytes(engine) / 1e9, 3),
+             "decode_graphs": bool(engine.core.executor.use_graphs), "step_program": engine.core.executor.program is not None}
+        for batch in (1, 8, 64):
+            dt, _ = decode_run(engine, batch, 512, args.steps, args.warmup, seed=batch)
+            m["decode_b%d_tok_s" % batch] = round(batch * args.steps / dt, 1)
+            m["decode_b%d_ms" % batch] = round(decode_run.median_ms, 3)
+        for n in (512, 2048):
+            t = prefill_run(engine, n, 5, seed=n)
+            m["prefill_%d_tok_s" % n] = round(n / t, 1)
+            m["prefill_%d_ms" % n] = round(t * 1e3, 3)
+        out["models"][name] = m
+        del engine
+        gc.collect()
+        torch.cuda.empty_cache()
+    t, l = out["models"]["takosun"], out["models"]["llama"]
+    out["takosun_over_llama"] = {k: round(t[k] / l[k], 3) for k in t if k.endswith("tok_s")}
+    out["value"], out["higher_is_better"] = t["decode_b8_tok_s"], True
+    print(json.dumps(out))
+
+
 def prefill_flops(cfg, T):
     """Multiply-adds times two of a causal prefill of T tokens: the linear layers on every token, the
     attention scores and values over the causal half, the LM head on one row."""
@@ -428,10 +487,12 @@ def main():
     ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products", "takosun"],
                     help="decode: the default line (Llama-3-8B shape); serve: continuous batching of 64 requests at "
                          "Llama-2-7B shape, a line of its own; products: a layer's matrix products alone, the "
-                         "library's against the engine's choice, at --rows")
+                         "library's against the engine's choice, at --rows; takosun: a Takosun model beside the Llama model "
+                         "of equal size, prefill and decode")
+    ap.add_argument("--takosun-sizes", default="2b", choices=["2b", "7b"], help="takosun: the layers' sizes")
     ap.add_argument("--rows", default="17,64,100,128,129,192,256,512,2048", help="products: numbers of rows")
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
@@ -466,6 +527,9 @@ def main():
         return
     if args.workload == "products":
         products_run(args)
+        return
+    if args.workload == "takosun":
+        takosun_run(args)
         return
     import torch
     shape_name, shape_cfg = SHAPES[args.shape]

@@ -43,7 +43,10 @@ int lmsf_rope_tail(const void* x, int dtype, long x_stride, int x_head, int x_at
 // moe.hip
 int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd, const int* ids,
     const int* table, int vocab, int top, int E, float weight, const void* base, long base_stride, void* act,
-    void* out, long out_stride, int n_tokens, int F, int W, hipStream_t stream);
+    void* out, long out_stride, int n_tokens, int F, int W, int* scratch_ints, float* scratch_rows,
+    hipStream_t stream);
+long lmsf_table_moe_scratch_ints(int n_tokens, int top, int E);
+int lmsf_table_moe_grouped(int dtype, int n_tokens, int top, int E, int F, int W, long h_stride);
 
 // blas.hip
 int lmsf_blas_init(long workspace_bytes);

@@ -4,8 +4,15 @@
 // The choice is read on the device from the step's token ids, so a step needs nothing from the host and can be
 // replayed from a graph. The experts' matrices lie stacked: Wgu [E, 2 F, W] (gate rows, then up rows), Wd [E, W, F].
 //
-// Few tokens (decoding): every (token, choice) streams its expert's rows, a wave per output, the token's vector in
-// LDS. Accumulation in float32.
+// Few tokens (decoding), and float32 at any number: every (token, choice) streams its expert's rows, a wave per
+// output, the token's vector in LDS, 16-byte loads where the rows allow them.
+// Many tokens in bfloat16: the (token, choice) pairs are grouped by expert on the device (one small kernel: counts,
+// offsets, an order, a list of tiles of up to 64 pairs of one expert), and each tile runs on the matrix cores
+// against a block of its expert's rows: A = 16 rows of W x 32 k, B = 16 pairs x 32 k, four tiles of pairs and, in the
+// gated product, the gate and the up rows of the same 16 outputs a wave, operands straight from memory. The down
+// product leaves float32 rows per pair; a last kernel adds a token's pairs and the shared part. A pair's result
+// does not depend on where in its tile it lies, so the order inside an expert's group (atomic counters) is free.
+// Accumulation in float32 throughout.
 #include "common.h"
 
 #include <math.h>
@@ -14,11 +21,30 @@
 #define MOE_WAVES (MOE_THREADS / LMSF_WAVE)
 #define MOE_OUT_PER_WAVE 4
 
+// sum_i w[i] x[i] over a row of W entries, the lanes of a wave together; x in LDS as float32
+template <typename T>
+__device__ __forceinline__ float moe_row_dot(const T* __restrict__ w, const float* __restrict__ x, int W, int lane,
+                                             bool vec) {
+  float a = 0.f;
+  if (vec) {
+    constexpr int V = Vec16<T>::N;
+    for (int i = lane * V; i < W; i += LMSF_WAVE * V) {
+      Vec16<T> p;
+      p.load(w + i);
+#pragma unroll
+      for (int e = 0; e < V; ++e) a += p.get(e) * x[i + e];
+    }
+  } else {
+    for (int i = lane; i < W; i += LMSF_WAVE) a += to_f32<T>(w[i]) * x[i];
+  }
+  return wave_sum(a);
+}
+
 // act[(n * top + k), f] = silu(Wg_e[f] . h[n]) * (Wu_e[f] . h[n]),  e = table[ids[n], k]
 template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
     const T* __restrict__ h, long h_stride, const T* __restrict__ Wgu, const int* __restrict__ ids,
-    const int* __restrict__ table, int vocab, int top, int E, T* __restrict__ act, int F, int W) {
+    const int* __restrict__ table, int vocab, int top, int E, T* __restrict__ act, int F, int W, int vec) {
   extern __shared__ float sh[];   // [W]
   const int nk = blockIdx.x, n = nk / top, k = nk - n * top;
   const int id = min(max(ids[n], 0), vocab - 1);
@@ -31,14 +57,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
   for (int f = f0; f < min(F, f0 + MOE_OUT_PER_WAVE); ++f) {
     const T* g = We + (long)f * W;
     const T* u = We + (long)(F + f) * W;
-    float ag = 0.f, au = 0.f;
-    for (int i = lane; i < W; i += LMSF_WAVE) {
-      const float x = sh[i];
-      ag += to_f32<T>(g[i]) * x;
-      au += to_f32<T>(u[i]) * x;
-    }
-    ag = wave_sum(ag);
-    au = wave_sum(au);
+    const float ag = moe_row_dot<T>(g, sh, W, lane, vec), au = moe_row_dot<T>(u, sh, W, lane, vec);
     if (lane == 0) {
       // the two products are rounded as stored activations are, then the activation in float32
       const float gg = to_f32<T>(from_f32<T>(ag)), uu = to_f32<T>(from_f32<T>(au));
@@ -52,7 +71,7 @@ template <typename T>
 __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
     const T* __restrict__ act, const T* __restrict__ Wd, const int* __restrict__ ids, const int* __restrict__ table,
     int vocab, int top, int E, float weight, const T* __restrict__ base, long base_stride, T* __restrict__ out,
-    long out_stride, int F, int W) {
+    long out_stride, int F, int W, int vec) {
   extern __shared__ float sa[];   // [top, F]
   const int n = blockIdx.x;
   const int id = min(max(ids[n], 0), vocab - 1);
@@ -65,9 +84,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
     for (int k = 0; k < top; ++k) {
       const int e = min(max(table[(long)id * top + k], 0), E - 1);
       const T* wr = Wd + ((long)e * W + o) * F;
-      float a = 0.f;
-      for (int i = lane; i < F; i += LMSF_WAVE) a += to_f32<T>(wr[i]) * sa[k * F + i];
-      total += wave_sum(a);
+      total += moe_row_dot<T>(wr, sa + k * F, F, lane, vec);
     }
     if (lane == 0) {
       const float b = base ? to_f32<T>(base[(long)n * base_stride + o]) : 0.f;
@@ -76,10 +93,139 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
   }
 }
 
+// ---------------------------------------------------------------- many tokens: grouped by expert, matrix cores
+
+#define MOE_TILE 64          // pairs a tile holds (four matrix-core tiles of 16)
+
+// Groups the P = N * top pairs by expert. order[i]: the pair at place i of the grouped sequence; tiles: for every
+// tile its expert, its first place and its number of pairs; n_tiles[0]: how many tiles there are. One workgroup.
+__global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, const int* __restrict__ table,
+                                                        int vocab, int top, int E, int P, int* __restrict__ order,
+                                                        int* __restrict__ tiles, int* __restrict__ n_tiles) {
+  extern __shared__ int sm[];   // [E] counts, [E] first places, [E] fill counters
+  int* cnt = sm;
+  int* first = sm + E;
+  int* fill = sm + 2 * E;
+  for (int e = threadIdx.x; e < E; e += blockDim.x) cnt[e] = fill[e] = 0;
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int id = min(max(ids[p / top], 0), vocab - 1);
+    atomicAdd(&cnt[min(max(table[(long)id * top + p % top], 0), E - 1)], 1);
+  }
+  __syncthreads();
+  if (threadIdx.x == 0) {
+    int at = 0, t = 0;
+    for (int e = 0; e < E; ++e) {
+      first[e] = at;
+      for (int s = 0; s < cnt[e]; s += MOE_TILE) {
+        tiles[3 * t] = e;
+        tiles[3 * t + 1] = at + s;
+        tiles[3 * t + 2] = min(MOE_TILE, cnt[e] - s);
+        ++t;
+      }
+      at += cnt[e];
+    }
+    n_tiles[0] = t;
+  }
+  __syncthreads();
+  for (int p = threadIdx.x; p < P; p += blockDim.x) {
+    const int id = min(max(ids[p / top], 0), vocab - 1);
+    const int e = min(max(table[(long)id * top + p % top], 0), E - 1);
+    order[first[e] + atomicAdd(&fill[e], 1)] = p;
+  }
+}
+
+// One tile of pairs against 64 outputs of its expert. GATED: x = the tokens' vectors (row of pair p: p / top),
+// Wm = Wgu, K = W, O = F, y = act [P, F] bfloat16 = silu(gate) * up; else x = act (row of pair p: p), Wm = Wd, K = F,
+// O = W, y = float32 rows [P, W].
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict__ x, long x_stride, int top,
+                                                       const bf16_t* __restrict__ Wm, const int* __restrict__ order,
+                                                       const int* __restrict__ tiles, const int* __restrict__ n_tiles,
+                                                       void* __restrict__ y, int O, int K) {
+  const int t = blockIdx.x;
+  if (t >= n_tiles[0]) return;
+  const int e = tiles[3 * t], place = tiles[3 * t + 1], count = tiles[3 * t + 2];
+  const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
+  const int fr = lane % 16, fg = lane / 16;
+  const int o0 = blockIdx.y * 64 + wave * 16;
+  if (o0 >= O) return;
+  constexpr int NA = GATED ? 2 : 1;
+  const int orow = min(o0 + fr, O - 1);
+  const bf16_t* wa[NA];
+  wa[0] = Wm + ((long)e * (GATED ? 2 : 1) * O + orow) * K + fg * 8;
+  if (GATED) wa[NA - 1] = Wm + ((long)e * 2 * O + O + orow) * K + fg * 8;
+  const bf16_t* xb[4];
+  int pair[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    pair[mt] = order[place + min(mt * 16 + fr, count - 1)];
+    xb[mt] = x + (long)(GATED ? pair[mt] / top : pair[mt]) * x_stride + fg * 8;
+  }
+  f32x4_t acc[NA][4];
+#pragma unroll
+  for (int a = 0; a < NA; ++a)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[a][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < K; k += 32) {
+    bf16x8_t fa[NA], fb[4];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) fa[a] = *reinterpret_cast<const bf16x8_t*>(wa[a] + k);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) fb[mt] = *reinterpret_cast<const bf16x8_t*>(xb[mt] + k);
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[a], fb[mt], acc[a][mt], 0, 0, 0);
+  }
+  // lane: pair fr of every tile of pairs, outputs o0 + fg * 4 .. + 3
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    if (mt * 16 + fr >= count) continue;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int o = o0 + fg * 4 + j;
+      if (o >= O) continue;
+      if (GATED) {
+        const float g = bf16_to_f32(f32_to_bf16(acc[0][mt][j])), u = bf16_to_f32(f32_to_bf16(acc[NA - 1][mt][j]));
+        reinterpret_cast<bf16_t*>(y)[(long)pair[mt] * O + o] = f32_to_bf16(g / (1.f + expf(-g)) * u);
+      } else {
+        reinterpret_cast<float*>(y)[(long)pair[mt] * O + o] = acc[0][mt][j];
+      }
+    }
+  }
+}
+
+// out[n, o] = base[n, o] + weight * sum_k rows[n * top + k, o]
+__global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, int top, float weight,
+                                                          const bf16_t* __restrict__ base, long base_stride,
+                                                          bf16_t* __restrict__ out, long out_stride, int W) {
+  const int n = blockIdx.x;
+  for (int o = threadIdx.x; o < W; o += 256) {
+    float s = 0.f;
+    for (int k = 0; k < top; ++k) s += rows[((long)n * top + k) * W + o];
+    const float b = base ? bf16_to_f32(base[(long)n * base_stride + o]) : 0.f;
+    out[(long)n * out_stride + o] = f32_to_bf16(b + weight * s);
+  }
+}
+
+// ints and floats of scratch that the grouped form needs for n_tokens tokens
+extern "C" long lmsf_table_moe_scratch_ints(int n_tokens, int top, int E) {
+  const long P = (long)n_tokens * top;
+  return P + 3 * (P / MOE_TILE + E + 1) + 4;
+}
+
+// whether lmsf_table_moe takes the grouped form for these sizes (then it needs the scratch: ints as above,
+// floats n_tokens * top * W)
+extern "C" int lmsf_table_moe_grouped(int dtype, int n_tokens, int top, int E, int F, int W, long h_stride) {
+  return dtype == LMSF_BF16 && (long)n_tokens * top >= 32 && W % 32 == 0 && F % 32 == 0 && h_stride % 8 == 0 &&
+         E <= 4096;
+}
+
 extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, const void* Wd, const int* ids,
                               const int* table, int vocab, int top, int E, float weight, const void* base,
                               long base_stride, void* act, void* out, long out_stride, int n_tokens, int F, int W,
-                              hipStream_t stream) {
+                              int* scratch_ints, float* scratch_rows, hipStream_t stream) {
   LMSF_CHECK(h && Wgu && Wd && ids && table && act && out, "table_moe: null pointer");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "table_moe: unknown dtype code %d", dtype);
   LMSF_CHECK(vocab > 0 && top > 0 && E > 0 && F > 0 && W > 0, "table_moe: bad sizes");
@@ -87,20 +233,40 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
   LMSF_CHECK((size_t)W * 4 <= 64 * 1024 && (size_t)top * F * 4 <= 64 * 1024, "table_moe: a row does not fit LDS");
   LMSF_CHECK((long)n_tokens * top < 2147483647L, "table_moe: too many rows");
   if (n_tokens <= 0) return 0;
+  if (lmsf_table_moe_grouped(dtype, n_tokens, top, E, F, W, h_stride) && scratch_ints && scratch_rows &&
+      lmsf_aligned16(h) && lmsf_aligned16(Wgu) && lmsf_aligned16(Wd) && lmsf_aligned16(act)) {
+    const int P = n_tokens * top, max_tiles = P / MOE_TILE + E;
+    int* order = scratch_ints;
+    int* tiles = order + P;
+    int* n_tiles = tiles + 3 * (max_tiles + 1);
+    hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)3 * E * 4, stream, ids, table, vocab, top, E, P,
+                       order, tiles, n_tiles);
+    hipLaunchKernelGGL((moe_tile_kernel<true>), dim3(max_tiles, (F + 63) / 64), dim3(256), 0, stream, (const bf16_t*)h,
+                       h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
+    hipLaunchKernelGGL((moe_tile_kernel<false>), dim3(max_tiles, (W + 63) / 64), dim3(256), 0, stream,
+                       (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows, W,
+                       F);
+    hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, scratch_rows, top, weight,
+                       (const bf16_t*)base, base_stride, (bf16_t*)out, out_stride, W);
+    LMSF_LAUNCH_CHECK("table_moe (grouped)");
+    return 0;
+  }
   const int per_block = MOE_WAVES * MOE_OUT_PER_WAVE;
   const dim3 g1(n_tokens * top, (F + per_block - 1) / per_block), g2(n_tokens, (W + per_block - 1) / per_block);
+  const int es = lmsf_elem_size(dtype), vn = 16 / es;
+  const int vec1 = W % vn == 0 && lmsf_aligned16(Wgu), vec2 = F % vn == 0 && lmsf_aligned16(Wd);
   if (dtype == LMSF_F32) {
     hipLaunchKernelGGL((moe_gate_up_kernel<float>), g1, dim3(MOE_THREADS), (size_t)W * 4, stream, (const float*)h,
-                       h_stride, (const float*)Wgu, ids, table, vocab, top, E, (float*)act, F, W);
+                       h_stride, (const float*)Wgu, ids, table, vocab, top, E, (float*)act, F, W, vec1);
     hipLaunchKernelGGL((moe_down_kernel<float>), g2, dim3(MOE_THREADS), (size_t)top * F * 4, stream, (const float*)act,
                        (const float*)Wd, ids, table, vocab, top, E, weight, (const float*)base, base_stride,
-                       (float*)out, out_stride, F, W);
+                       (float*)out, out_stride, F, W, vec2);
   } else {
     hipLaunchKernelGGL((moe_gate_up_kernel<bf16_t>), g1, dim3(MOE_THREADS), (size_t)W * 4, stream, (const bf16_t*)h,
-                       h_stride, (const bf16_t*)Wgu, ids, table, vocab, top, E, (bf16_t*)act, F, W);
+                       h_stride, (const bf16_t*)Wgu, ids, table, vocab, top, E, (bf16_t*)act, F, W, vec1);
     hipLaunchKernelGGL((moe_down_kernel<bf16_t>), g2, dim3(MOE_THREADS), (size_t)top * F * 4, stream,
                        (const bf16_t*)act, (const bf16_t*)Wd, ids, table, vocab, top, E, weight, (const bf16_t*)base,
-                       base_stride, (bf16_t*)out, out_stride, F, W);
+                       base_stride, (bf16_t*)out, out_stride, F, W, vec2);
   }
   LMSF_LAUNCH_CHECK("table_moe");
   return 0;

@@ -710,10 +710,15 @@ class HipOps:
         vocab, top = table.shape
         act = torch.empty((N * top, F), dtype=h.dtype, device=h.device)
         out = torch.empty((N, W), dtype=h.dtype, device=h.device)
+        ints = rows = None
+        if self.lib.lmsf_table_moe_grouped(_code(h.dtype), N, top, E, F, W, h.stride(0)):
+            # many tokens: grouped by expert on the device, tiles on the matrix cores
+            ints = torch.empty(self.lib.lmsf_table_moe_scratch_ints(N, top, E), dtype=torch.int32, device=h.device)
+            rows = torch.empty((N * top, W), dtype=torch.float32, device=h.device)
         self._check(self.lib.lmsf_table_moe(
             _ptr(h), _code(h.dtype), h.stride(0), _ptr(w_gate_up), _ptr(w_down), _ptr(token_ids), _ptr(table), vocab,
             top, E, float(weight), _ptr(base), base.stride(0) if base is not None else 0, _ptr(act), _ptr(out),
-            out.stride(0), N, F, W, self._stream()))
+            out.stride(0), N, F, W, _ptr(ints), _ptr(rows), self._stream()))
         return out
 
     # ------------------------------------------------------------------ feed-forward

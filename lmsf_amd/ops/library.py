@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 24
+ABI_VERSION = 25
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -48,7 +48,9 @@ _SIGNATURES = {
     "lmsf_rope_tail": (c_int, [_P, c_int, c_long, c_int, c_int, _P, c_long, c_int, c_int, _P, _P, c_int, c_int, c_int,
                                c_int, c_int, _P]),
     "lmsf_table_moe": (c_int, [_P, c_int, c_long, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_long, _P, _P,
-                               c_long, c_int, c_int, c_int, _P]),
+                               c_long, c_int, c_int, c_int, _P, _P, _P]),
+    "lmsf_table_moe_scratch_ints": (c_long, [c_int, c_int, c_int]),
+    "lmsf_table_moe_grouped": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_long]),
     "lmsf_gated_act": (c_int, [_P, _P, c_int, c_int, c_int, c_long, c_int, _P]),
     "lmsf_gemm_plain": (c_int, [_P, c_int, c_long, _P, c_int, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, _P]),
     "lmsf_gemm_skinny": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P]),

@@ -155,11 +155,13 @@ def test_latent_rows_and_rotated_query_parts(dtype, R, dr, rot, D, ps):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("W,F,E,top,shared", [(64, 32, 3, 2, True), (120, 24, 5, 1, False), (32, 16, 6, 6, True), (256, 100, 4, 3, False)])
-def test_experts_assigned_by_a_table(dtype, W, F, E, top, shared):
+@pytest.mark.parametrize("N", [13, 150, 333])      # few tokens stream the experts' rows; many are grouped by expert
+@pytest.mark.parametrize("W,F,E,top,shared", [(64, 32, 3, 2, True), (120, 24, 5, 1, False), (32, 16, 6, 6, True),
+                                              (256, 100, 4, 3, False), (128, 96, 7, 2, True), (96, 64, 70, 1, False)])
+def test_experts_assigned_by_a_table(dtype, W, F, E, top, shared, N):
     o = ops()
     g = torch.Generator().manual_seed(W + F + E)
-    V, N = 37, 13
+    V = 37
     w = {}
     for e in range(E):
         w["m.e%d.gate" % e] = (torch.randn((F, W), generator=g) / math.sqrt(W)).to(dtype).float()

@@ -13,13 +13,14 @@
 //                                                           the results of all layers so far, r being the k-th)
 //   out[row] = wn ? gn(x; wn) : x                           the norm *before* the next sublayer
 //
-// All arithmetic is float32; branch and out are float32 or bfloat16, the weights float32. One workgroup of 256
-// threads a row, the row kept in LDS between the passes.
+// All arithmetic is float32; branch and out are float32 or bfloat16, the weights float32. One workgroup a row
+// (256 to 1,024 threads), the row kept in LDS between the passes.
 #include "common.h"
 
 #include <math.h>
 
-#define GN_THREADS 256
+#define GN_MAX_THREADS 1024
+#define GN_THREADS ((int)blockDim.x)
 
 template <typename T>
 __device__ __forceinline__ float gn_load(const void* p, long i) { return to_f32<T>(((const T*)p)[i]); }
@@ -42,7 +43,7 @@ __device__ __forceinline__ void gn_normalize(float* row, const float* __restrict
 }
 
 template <typename TB, typename TO>
-__global__ __launch_bounds__(GN_THREADS) void group_norm_kernel(
+__global__ __launch_bounds__(GN_MAX_THREADS) void group_norm_kernel(
     const TB* __restrict__ branch, long branch_stride, const float* __restrict__ wb, float* __restrict__ residual,
     float* __restrict__ hist, long hist_stride, int hist_index, const float* __restrict__ mix,
     const float* __restrict__ wn, TO* __restrict__ out, long out_stride, const int* __restrict__ rows, int W,
@@ -87,7 +88,10 @@ static void gn_launch(int n_rows, size_t smem, hipStream_t stream, const void* b
                       const float* wb, float* residual, float* hist, long hist_stride, int hist_index,
                       const float* mix, const float* wn, void* out, long out_stride, const int* rows, int W,
                       int groups, float eps_b, float eps_n) {
-  hipLaunchKernelGGL((group_norm_kernel<TB, TO>), dim3(n_rows), dim3(GN_THREADS), smem, stream, (const TB*)branch,
+  // few rows: a row's passes wait for memory one after the other, so many threads with few elements each; many
+  // rows fill the chip with smaller workgroups
+  const int threads = n_rows >= 1024 || W <= 256 ? 256 : W <= 1024 ? 512 : 1024;
+  hipLaunchKernelGGL((group_norm_kernel<TB, TO>), dim3(n_rows), dim3(threads), smem, stream, (const TB*)branch,
                      branch_stride, wb, residual, hist, hist_stride, hist_index, mix, wn, (TO*)out, out_stride, rows,
                      W, groups, eps_b, eps_n);
 }

@@ -10,6 +10,7 @@
 //
 //   lmsf_latent_cache_write   c = rms_norm(x[:R]) * w, r = rotate(x[R:R+dr]) -> pages at the token's slot
 //   lmsf_head_linear          y[n, h, :] = W_h x[n, h, :K] (* sigmoid(gate[n, h])), W [H, O, K]: per-head products
+//                             (32 tokens and more in bfloat16: on the matrix cores)
 //   lmsf_rope_tail            rotates one part of every head of q into another buffer and zeroes its padding
 //
 // Norm, rotation, gate and accumulation are float32; storage is float32 or bfloat16.
@@ -100,7 +101,7 @@ extern "C" int lmsf_latent_cache_write(const void* x, int dtype, long x_stride, 
 template <typename T>
 __global__ __launch_bounds__(LAT_THREADS) void head_linear_kernel(
     const T* __restrict__ x, long x_stride, int x_head, const T* __restrict__ W, T* __restrict__ y, long y_stride,
-    int y_head, const T* __restrict__ gate, long gate_stride, int n_tokens, int O, int K) {
+    int y_head, const T* __restrict__ gate, long gate_stride, int n_tokens, int O, int K, int vec) {
   extern __shared__ float sx[];   // [HL_TOKENS, K]
   const int h = blockIdx.y, n0 = blockIdx.x * HL_TOKENS;
   const int nt = min(HL_TOKENS, n_tokens - n0);
@@ -116,19 +117,77 @@ __global__ __launch_bounds__(LAT_THREADS) void head_linear_kernel(
     if (gate && t < nt) g[t] = 1.f / (1.f + expf(-to_f32<T>(gate[(long)(n0 + t) * gate_stride + h])));
   }
   const T* Wh = W + (long)h * O * K;
+  constexpr int V = Vec16<T>::N;
   for (int o = threadIdx.x; o < O; o += LAT_THREADS) {
     float acc[HL_TOKENS];
 #pragma unroll
     for (int t = 0; t < HL_TOKENS; ++t) acc[t] = 0.f;
     const T* wr = Wh + (long)o * K;
-    for (int k = 0; k < K; ++k) {
-      const float wv = to_f32<T>(wr[k]);
+    if (vec) {
+      // 16 bytes of a row of W a load
+      for (int k = 0; k < K; k += V) {
+        Vec16<T> p;
+        p.load(wr + k);
 #pragma unroll
-      for (int t = 0; t < HL_TOKENS; ++t) acc[t] += wv * sx[t * K + k];
+        for (int e = 0; e < V; ++e) {
+          const float wv = p.get(e);
+#pragma unroll
+          for (int t = 0; t < HL_TOKENS; ++t) acc[t] += wv * sx[t * K + k + e];
+        }
+      }
+    } else {
+      for (int k = 0; k < K; ++k) {
+        const float wv = to_f32<T>(wr[k]);
+#pragma unroll
+        for (int t = 0; t < HL_TOKENS; ++t) acc[t] += wv * sx[t * K + k];
+      }
     }
 #pragma unroll
     for (int t = 0; t < HL_TOKENS; ++t)
       if (t < nt) y[(long)(n0 + t) * y_stride + (long)h * y_head + o] = from_f32<T>(acc[t] * g[t]);
+  }
+}
+
+// The same product on the matrix cores, for many tokens in bfloat16: a workgroup takes 64 tokens of one head against
+// 64 outputs, a wave 16 of the outputs (A = 16 rows of W_h x 32 k) and four tiles of 16 tokens (B), operands straight
+// from memory. K is a multiple of 32; rows and heads begin at multiples of 16 bytes.
+__global__ __launch_bounds__(256) void head_linear_mfma_kernel(
+    const bf16_t* __restrict__ x, long x_stride, int x_head, const bf16_t* __restrict__ W, bf16_t* __restrict__ y,
+    long y_stride, int y_head, const bf16_t* __restrict__ gate, long gate_stride, int n_tokens, int O, int K) {
+  const int h = blockIdx.y, n0 = blockIdx.x * 64;
+  const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
+  const int fr = lane % 16, fg = lane / 16;
+  const int o0 = blockIdx.z * 64 + wave * 16;
+  if (o0 >= O) return;
+  const bf16_t* wa = W + ((long)h * O + min(o0 + fr, O - 1)) * K + fg * 8;
+  const bf16_t* xb[4];
+  int tok[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    tok[mt] = n0 + mt * 16 + fr;
+    xb[mt] = x + (long)min(tok[mt], n_tokens - 1) * x_stride + (long)h * x_head + fg * 8;
+  }
+  f32x4_t acc[4];
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  for (int k = 0; k < K; k += 32) {
+    const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(wa + k);
+    bf16x8_t fb[4];
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) fb[mt] = *reinterpret_cast<const bf16x8_t*>(xb[mt] + k);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa, fb[mt], acc[mt], 0, 0, 0);
+  }
+  // lane: token fr of every tile of tokens, outputs o0 + fg * 4 .. + 3
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    if (tok[mt] >= n_tokens) continue;
+    const float g = gate ? 1.f / (1.f + expf(-bf16_to_f32(gate[(long)tok[mt] * gate_stride + h]))) : 1.f;
+#pragma unroll
+    for (int j = 0; j < 4; ++j) {
+      const int o = o0 + fg * 4 + j;
+      if (o < O) y[(long)tok[mt] * y_stride + (long)h * y_head + o] = f32_to_bf16(acc[mt][j] * g);
+    }
   }
 }
 
@@ -142,16 +201,26 @@ extern "C" int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_h
   LMSF_CHECK(x_stride >= (long)(H - 1) * x_head + K && y_stride >= (long)(H - 1) * y_head + O, "head_linear: rows overlap");
   LMSF_CHECK((size_t)HL_TOKENS * K * 4 <= 64 * 1024, "head_linear: %d inputs a head do not fit LDS", K);
   if (n_tokens <= 0) return 0;
+  const int es = lmsf_elem_size(dtype);
+  const bool rows16 = lmsf_aligned16(x) && lmsf_aligned16(W) && (x_stride * es) % 16 == 0 && ((long)x_head * es) % 16 == 0;
+  if (dtype == LMSF_BF16 && n_tokens >= 32 && K % 32 == 0 && rows16) {
+    hipLaunchKernelGGL(head_linear_mfma_kernel, dim3((n_tokens + 63) / 64, H, (O + 63) / 64), dim3(256), 0, stream,
+                       (const bf16_t*)x, x_stride, x_head, (const bf16_t*)W, (bf16_t*)y, y_stride, y_head,
+                       (const bf16_t*)gate, gate_stride, n_tokens, O, K);
+    LMSF_LAUNCH_CHECK("head_linear (matrix cores)");
+    return 0;
+  }
+  const int vec = lmsf_aligned16(W) && (K * es) % 16 == 0;
   const dim3 grid((n_tokens + HL_TOKENS - 1) / HL_TOKENS, H);
   const size_t smem = (size_t)HL_TOKENS * K * 4;
   if (dtype == LMSF_F32)
     hipLaunchKernelGGL((head_linear_kernel<float>), grid, dim3(LAT_THREADS), smem, stream, (const float*)x, x_stride,
                        x_head, (const float*)W, (float*)y, y_stride, y_head, (const float*)gate, gate_stride, n_tokens,
-                       O, K);
+                       O, K, vec);
   else
     hipLaunchKernelGGL((head_linear_kernel<bf16_t>), grid, dim3(LAT_THREADS), smem, stream, (const bf16_t*)x, x_stride,
                        x_head, (const bf16_t*)W, (bf16_t*)y, y_stride, y_head, (const bf16_t*)gate, gate_stride,
-                       n_tokens, O, K);
+                       n_tokens, O, K, vec);
   LMSF_LAUNCH_CHECK("head_linear");
   return 0;
 }

@@ -135,7 +135,7 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   }
 }
 
-// One tile of pairs against 64 outputs of its expert. GATED: x = the tokens' vectors (row of pair p: p / top),
+// One tile of pairs against 128 outputs of its expert (32 a wave). GATED: x = the tokens' vectors (row of pair p: p / top),
 // Wm = Wgu, K = W, O = F, y = act [P, F] bfloat16 = silu(gate) * up; else x = act (row of pair p: p), Wm = Wd, K = F,
 // O = W, y = float32 rows [P, W].
 template <bool GATED>
@@ -148,13 +148,17 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
   const int e = tiles[3 * t], place = tiles[3 * t + 1], count = tiles[3 * t + 2];
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int fr = lane % 16, fg = lane / 16;
-  const int o0 = blockIdx.y * 64 + wave * 16;
+  constexpr int NO = 2;                    // tiles of 16 outputs a wave
+  constexpr int NA = GATED ? 2 * NO : NO;  // tiles of rows of W a wave: gate and up rows of the same outputs
+  const int o0 = blockIdx.y * (64 * NO) + wave * (16 * NO);
   if (o0 >= O) return;
-  constexpr int NA = GATED ? 2 : 1;
-  const int orow = min(o0 + fr, O - 1);
   const bf16_t* wa[NA];
-  wa[0] = Wm + ((long)e * (GATED ? 2 : 1) * O + orow) * K + fg * 8;
-  if (GATED) wa[NA - 1] = Wm + ((long)e * 2 * O + O + orow) * K + fg * 8;
+#pragma unroll
+  for (int a = 0; a < NO; ++a) {
+    const int orow = min(o0 + a * 16 + fr, O - 1);
+    wa[a] = Wm + ((long)e * (GATED ? 2 : 1) * O + orow) * K + fg * 8;
+    if (GATED) wa[NO + a] = Wm + ((long)e * 2 * O + O + orow) * K + fg * 8;
+  }
   const bf16_t* xb[4];
   int pair[4];
 #pragma unroll
@@ -178,21 +182,23 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[a], fb[mt], acc[a][mt], 0, 0, 0);
   }
-  // lane: pair fr of every tile of pairs, outputs o0 + fg * 4 .. + 3
+  // lane: pair fr of every tile of pairs, outputs o0 + a * 16 + fg * 4 .. + 3
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
     if (mt * 16 + fr >= count) continue;
 #pragma unroll
-    for (int j = 0; j < 4; ++j) {
-      const int o = o0 + fg * 4 + j;
-      if (o >= O) continue;
-      if (GATED) {
-        const float g = bf16_to_f32(f32_to_bf16(acc[0][mt][j])), u = bf16_to_f32(f32_to_bf16(acc[NA - 1][mt][j]));
-        reinterpret_cast<bf16_t*>(y)[(long)pair[mt] * O + o] = f32_to_bf16(g / (1.f + expf(-g)) * u);
-      } else {
-        reinterpret_cast<float*>(y)[(long)pair[mt] * O + o] = acc[0][mt][j];
+    for (int a = 0; a < NO; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int o = o0 + a * 16 + fg * 4 + j;
+        if (o >= O) continue;
+        if (GATED) {
+          const float g = bf16_to_f32(f32_to_bf16(acc[a][mt][j])), u = bf16_to_f32(f32_to_bf16(acc[NA - NO + a][mt][j]));
+          reinterpret_cast<bf16_t*>(y)[(long)pair[mt] * O + o] = f32_to_bf16(g / (1.f + expf(-g)) * u);
+        } else {
+          reinterpret_cast<float*>(y)[(long)pair[mt] * O + o] = acc[a][mt][j];
+        }
       }
-    }
   }
 }
 
@@ -241,9 +247,9 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
     int* n_tiles = tiles + 3 * (max_tiles + 1);
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)3 * E * 4, stream, ids, table, vocab, top, E, P,
                        order, tiles, n_tiles);
-    hipLaunchKernelGGL((moe_tile_kernel<true>), dim3(max_tiles, (F + 63) / 64), dim3(256), 0, stream, (const bf16_t*)h,
+    hipLaunchKernelGGL((moe_tile_kernel<true>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream, (const bf16_t*)h,
                        h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
-    hipLaunchKernelGGL((moe_tile_kernel<false>), dim3(max_tiles, (W + 63) / 64), dim3(256), 0, stream,
+    hipLaunchKernelGGL((moe_tile_kernel<false>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
                        (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows, W,
                        F);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, scratch_rows, top, weight,

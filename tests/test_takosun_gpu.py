@@ -92,11 +92,12 @@ def test_group_norm_in_every_arrangement(dtype, W, groups):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("H,O,K,xh,oh", [(2, 32, 16, 24, 48), (5, 40, 24, 40, 56), (1, 300, 7, 7, 300), (3, 8, 513, 520, 8)])
+@pytest.mark.parametrize("H,O,K,xh,oh", [(2, 32, 16, 24, 48), (5, 40, 24, 40, 56), (1, 300, 7, 7, 300), (3, 8, 513, 520, 8),
+                                         (4, 40, 64, 96, 48), (3, 224, 32, 40, 256), (2, 70, 96, 96, 72)])
 def test_per_head_products_with_and_without_gate(dtype, H, O, K, xh, oh):
     o = ops()
     g = torch.Generator().manual_seed(H * O + K)
-    for N in (1, 8, 19):
+    for N in (1, 8, 19, 70, 200):          # from 32 tokens on, bfloat16 products with K a multiple of 32 use the matrix cores
         x = torch.randn((N, H * xh + 4), generator=g).to(dtype)
         W = (torch.randn((H, O, K), generator=g) / math.sqrt(K)).to(dtype)
         gate = torch.randn((N, H + 3), generator=g).to(dtype)

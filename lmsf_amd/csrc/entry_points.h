@@ -33,9 +33,11 @@ int lmsf_group_norm(const void* branch, int branch_dtype, long branch_stride, co
 // latent.hip
 int lmsf_latent_cache_write(const void* x, int dtype, long x_stride, const float* w, float eps, const int* positions,
     const float* table, int rot, int max_pos, const int* slots, void* k_pages, void* v_pages, long num_pages,
-    int n_tokens, int R, int dr, int D, int ps, hipStream_t stream);
+    int n_tokens, int R, int dr, int D, int ps, const void* qx, const float* qw, void* q_out, long q_out_stride,
+    int Q, hipStream_t stream);
 int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_head, const void* W, void* y, long y_stride,
-    int y_head, const void* gate, long gate_stride, int n_tokens, int H, int O, int K, hipStream_t stream);
+    int y_head, const void* gate, long gate_stride, int n_tokens, int H, int O, int K, const int* positions,
+    const float* table, int rot, int max_pos, int x_at, int y_at, int dr, hipStream_t stream);
 int lmsf_rope_tail(const void* x, int dtype, long x_stride, int x_head, int x_at, void* y, long y_stride, int y_head,
     int y_at, const int* positions, const float* table, int rot, int max_pos, int n_tokens, int H, int dr,
     hipStream_t stream);

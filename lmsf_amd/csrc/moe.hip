@@ -21,23 +21,37 @@
 #define MOE_WAVES (MOE_THREADS / LMSF_WAVE)
 #define MOE_OUT_PER_WAVE 4
 
-// sum_i w[i] x[i] over a row of W entries, the lanes of a wave together; x in LDS as float32
-template <typename T>
-__device__ __forceinline__ float moe_row_dot(const T* __restrict__ w, const float* __restrict__ x, int W, int lane,
-                                             bool vec) {
-  float a = 0.f;
+// NR rows of a matrix against one vector: out[r] = sum_i w[r * ld + i] x[i] over W entries, the lanes of a wave
+// together; x in LDS as float32. The loads of all rows are asked for before any is used (rows beyond ``valid`` repeat
+// the last valid one).
+template <typename T, int NR>
+__device__ __forceinline__ void moe_rows_dot(const T* __restrict__ w, long ld, int valid, const float* __restrict__ x,
+                                             int W, int lane, bool vec, float* out) {
+  float a[NR];
+#pragma unroll
+  for (int r = 0; r < NR; ++r) a[r] = 0.f;
   if (vec) {
     constexpr int V = Vec16<T>::N;
     for (int i = lane * V; i < W; i += LMSF_WAVE * V) {
-      Vec16<T> p;
-      p.load(w + i);
+      Vec16<T> p[NR];
 #pragma unroll
-      for (int e = 0; e < V; ++e) a += p.get(e) * x[i + e];
+      for (int r = 0; r < NR; ++r) p[r].load(w + (long)min(r, valid - 1) * ld + i);
+#pragma unroll
+      for (int e = 0; e < V; ++e) {
+        const float xv = x[i + e];
+#pragma unroll
+        for (int r = 0; r < NR; ++r) a[r] += p[r].get(e) * xv;
+      }
     }
   } else {
-    for (int i = lane; i < W; i += LMSF_WAVE) a += to_f32<T>(w[i]) * x[i];
+    for (int i = lane; i < W; i += LMSF_WAVE) {
+      const float xv = x[i];
+#pragma unroll
+      for (int r = 0; r < NR; ++r) a[r] += to_f32<T>(w[(long)min(r, valid - 1) * ld + i]) * xv;
+    }
   }
-  return wave_sum(a);
+#pragma unroll
+  for (int r = 0; r < NR; ++r) out[r] = wave_sum(a[r]);
 }
 
 // act[(n * top + k), f] = silu(Wg_e[f] . h[n]) * (Wu_e[f] . h[n]),  e = table[ids[n], k]
@@ -54,15 +68,21 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_gate_up_kernel(
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int f0 = (blockIdx.y * MOE_WAVES + wave) * MOE_OUT_PER_WAVE;
   const T* We = Wgu + (long)e * 2 * F * W;
-  for (int f = f0; f < min(F, f0 + MOE_OUT_PER_WAVE); ++f) {
-    const T* g = We + (long)f * W;
-    const T* u = We + (long)(F + f) * W;
-    const float ag = moe_row_dot<T>(g, sh, W, lane, vec), au = moe_row_dot<T>(u, sh, W, lane, vec);
-    if (lane == 0) {
-      // the two products are rounded as stored activations are, then the activation in float32
-      const float gg = to_f32<T>(from_f32<T>(ag)), uu = to_f32<T>(from_f32<T>(au));
-      act[(long)nk * F + f] = from_f32<T>(gg / (1.f + expf(-gg)) * uu);
-    }
+  if (f0 >= F) return;
+  const int valid = min(MOE_OUT_PER_WAVE, F - f0);
+  float ag[MOE_OUT_PER_WAVE], au[MOE_OUT_PER_WAVE];
+  moe_rows_dot<T, MOE_OUT_PER_WAVE>(We + (long)f0 * W, W, valid, sh, W, lane, vec, ag);
+  moe_rows_dot<T, MOE_OUT_PER_WAVE>(We + (long)(F + f0) * W, W, valid, sh, W, lane, vec, au);
+  if (lane < valid) {
+    // the two products are rounded as stored activations are, then the activation in float32
+    float gg = 0.f, uu = 0.f;
+#pragma unroll
+    for (int r = 0; r < MOE_OUT_PER_WAVE; ++r)
+      if (r == lane) {
+        gg = to_f32<T>(from_f32<T>(ag[r]));
+        uu = to_f32<T>(from_f32<T>(au[r]));
+      }
+    act[(long)nk * F + f0 + lane] = from_f32<T>(gg / (1.f + expf(-gg)) * uu);
   }
 }
 
@@ -79,17 +99,25 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
   __syncthreads();
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int o0 = (blockIdx.y * MOE_WAVES + wave) * MOE_OUT_PER_WAVE;
-  for (int o = o0; o < min(W, o0 + MOE_OUT_PER_WAVE); ++o) {
-    float total = 0.f;
-    for (int k = 0; k < top; ++k) {
-      const int e = min(max(table[(long)id * top + k], 0), E - 1);
-      const T* wr = Wd + ((long)e * W + o) * F;
-      total += moe_row_dot<T>(wr, sa + k * F, F, lane, vec);
-    }
-    if (lane == 0) {
-      const float b = base ? to_f32<T>(base[(long)n * base_stride + o]) : 0.f;
-      out[(long)n * out_stride + o] = from_f32<T>(b + weight * total);
-    }
+  if (o0 >= W) return;
+  const int valid = min(MOE_OUT_PER_WAVE, W - o0);
+  float total[MOE_OUT_PER_WAVE];
+#pragma unroll
+  for (int r = 0; r < MOE_OUT_PER_WAVE; ++r) total[r] = 0.f;
+  for (int k = 0; k < top; ++k) {
+    const int e = min(max(table[(long)id * top + k], 0), E - 1);
+    float part[MOE_OUT_PER_WAVE];
+    moe_rows_dot<T, MOE_OUT_PER_WAVE>(Wd + ((long)e * W + o0) * F, F, valid, sa + k * F, F, lane, vec, part);
+#pragma unroll
+    for (int r = 0; r < MOE_OUT_PER_WAVE; ++r) total[r] += part[r];
+  }
+  if (lane < valid) {
+    float mine = 0.f;
+#pragma unroll
+    for (int r = 0; r < MOE_OUT_PER_WAVE; ++r)
+      if (r == lane) mine = total[r];
+    const float b = base ? to_f32<T>(base[(long)n * base_stride + o0 + lane]) : 0.f;
+    out[(long)n * out_stride + o0 + lane] = from_f32<T>(b + weight * mine);
   }
 }
 

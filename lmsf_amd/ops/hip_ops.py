@@ -625,12 +625,22 @@ class HipOps:
 
     def latent_cache_write(self, x: torch.Tensor, weight: torch.Tensor, eps: float, rank: int, rot_width: int,
                            positions: torch.Tensor, table: torch.Tensor, slots: torch.Tensor, k_pages: torch.Tensor,
-                           v_pages: torch.Tensor) -> None:
+                           v_pages: torch.Tensor, also_norm: Optional[torch.Tensor] = None,
+                           also_weight: Optional[torch.Tensor] = None) -> Optional[torch.Tensor]:
         """Per token: c = rms_norm(x[:rank]) * weight, r = rotate(x[rank:rank + rot_width]) by the token's position
         (``table`` float32 [max_pos, rot] = [cos | sin], the first ``rot`` entries of r in pairs (i, i + rot/2));
         [c | r | zeros] goes to the token's slot of ``k_pages`` [pages, 1, page_size, D] and of ``v_pages``
-        [pages, 1, D, page_size]. A negative slot stores nothing."""
-        self._dev(x, weight, positions, table, slots, k_pages, v_pages)
+        [pages, 1, D, page_size]. A negative slot stores nothing. ``also_norm``: another view of the same rows (same
+        row stride) whose plain RMS norm with ``also_weight`` and the same eps is returned, from the same launch."""
+        self._dev(x, weight, positions, table, slots, k_pages, v_pages, also_norm, also_weight)
+        q_out = None
+        if also_norm is not None:
+            if also_norm.stride(0) != x.stride(0) or also_norm.stride(1) != 1 or also_norm.shape[0] != x.shape[0] \
+                    or also_norm.dtype != x.dtype or also_weight is None or also_weight.dtype != torch.float32 \
+                    or also_weight.shape != (also_norm.shape[1],) or not also_weight.is_contiguous():
+                raise ValueError("latent_cache_write: the second norm's operand must be a view of the same rows, its "
+                                 "weight contiguous float32")
+            q_out = torch.empty(tuple(also_norm.shape), dtype=x.dtype, device=x.device)
         N = x.shape[0]
         if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < rank + rot_width:
             raise ValueError("latent_cache_write: x must be [N, >= %d] with unit column stride" % (rank + rot_width))
@@ -651,14 +661,26 @@ class HipOps:
         self._check(self.lib.lmsf_latent_cache_write(
             _ptr(x), _code(x.dtype), x.stride(0), _ptr(weight), float(eps), _ptr(positions), _ptr(table),
             table.shape[1], table.shape[0], _ptr(slots), _ptr(k_pages), _ptr(v_pages), P, N, int(rank), int(rot_width),
-            D, ps, self._stream()))
+            D, ps, _ptr(also_norm), _ptr(also_weight), _ptr(q_out), q_out.stride(0) if q_out is not None else 0,
+            also_norm.shape[1] if also_norm is not None else 0, self._stream()))
+        return q_out
 
     def head_linear(self, x: torch.Tensor, x_head: int, weight: torch.Tensor, out: torch.Tensor, out_head: int,
-                    gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+                    gate: Optional[torch.Tensor] = None, rope_tail=None) -> torch.Tensor:
         """Per-head products: out[n, h * out_head + o] = sum_k weight[h, o, k] x[n, h * x_head + k], times
         sigmoid(gate[n, h]) if a gate is given. ``weight`` contiguous [H, O, K]; x, out and gate are views with
-        unit column stride whose first column is head 0's first entry."""
+        unit column stride whose first column is head 0's first entry. ``rope_tail`` = (x_at, out_at, width,
+        positions, table): also what ``rope_tail`` does with these arguments, from the same launch where it can be."""
         self._dev(x, weight, out, gate)
+        x_at = out_at = width = rot = max_pos = 0
+        positions = table = None
+        if rope_tail is not None:
+            x_at, out_at, width, positions, table = rope_tail
+            self._dev(positions, table)
+            if table.dtype != torch.float32 or table.dim() != 2 or not table.is_contiguous() or table.shape[1] > width:
+                raise ValueError("head_linear: bad rotary table")
+            self._i32(positions, "positions", x.shape[0])
+            rot, max_pos = table.shape[1], table.shape[0]
         H, O, K = weight.shape
         N = x.shape[0]
         if not weight.is_contiguous() or weight.dtype != x.dtype or out.dtype != x.dtype:
@@ -670,7 +692,8 @@ class HipOps:
             raise ValueError("head_linear: gate must be [N, >= %d] of x's dtype" % H)
         self._check(self.lib.lmsf_head_linear(
             _ptr(x), _code(x.dtype), x.stride(0), int(x_head), _ptr(weight), _ptr(out), out.stride(0), int(out_head),
-            _ptr(gate), gate.stride(0) if gate is not None else 0, N, H, O, K, self._stream()))
+            _ptr(gate), gate.stride(0) if gate is not None else 0, N, H, O, K, _ptr(positions), _ptr(table), rot, max_pos,
+            int(x_at), int(out_at), int(width), self._stream()))
         return out
 
     def rope_tail(self, x: torch.Tensor, x_head: int, x_at: int, out: torch.Tensor, out_head: int, out_at: int,

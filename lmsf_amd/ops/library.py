@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 25
+ABI_VERSION = 26
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -42,9 +42,9 @@ _SIGNATURES = {
     "lmsf_group_norm": (c_int, [_P, c_int, c_long, _P, _P, _P, c_long, c_int, _P, _P, _P, c_int, c_long, _P, c_int, c_int,
                                 c_int, c_float, c_float, _P]),
     "lmsf_latent_cache_write": (c_int, [_P, c_int, c_long, _P, c_float, _P, _P, c_int, c_int, _P, _P, _P, c_long, c_int,
-                                        c_int, c_int, c_int, c_int, _P]),
+                                        c_int, c_int, c_int, c_int, _P, _P, _P, c_long, c_int, _P]),
     "lmsf_head_linear": (c_int, [_P, c_int, c_long, c_int, _P, _P, c_long, c_int, _P, c_long, c_int, c_int, c_int, c_int,
-                                 _P]),
+                                 _P, _P, c_int, c_int, c_int, c_int, c_int, _P]),
     "lmsf_rope_tail": (c_int, [_P, c_int, c_long, c_int, c_int, _P, c_long, c_int, c_int, _P, _P, c_int, c_int, c_int,
                                c_int, c_int, _P]),
     "lmsf_table_moe": (c_int, [_P, c_int, c_long, _P, _P, _P, _P, c_int, c_int, c_int, c_float, _P, c_long, _P, _P,

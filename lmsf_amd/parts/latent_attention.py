@@ -97,12 +97,17 @@ class LatentAttention(Mixer):
         if binding.writes_cache:
             if not self.owns_latent:
                 raise ValueError("%s has no latent of its own to store" % self.prefix)
-            ops.latent_cache_write(low[:, self.at_kv:], self.kv_norm.weight, self.eps, self.R, self.dr, ctx.positions,
-                                   table, group.slots, binding.k_pages, binding.v_pages)
-        q = self.uq.forward(self.q_norm.forward(low[:, :self.Q]))            # [N, H (dn + dr)]
+            # the key/value latent into the pages and the query latent's norm, one launch
+            cq = ops.latent_cache_write(low[:, self.at_kv:], self.kv_norm.weight, self.eps, self.R, self.dr, ctx.positions,
+                                        table, group.slots, binding.k_pages, binding.v_pages,
+                                        also_norm=low[:, :self.Q], also_weight=self.q_norm.weight)
+        else:
+            cq = self.q_norm.forward(low[:, :self.Q])
+        q = self.uq.forward(cq)                                              # [N, H (dn + dr)]
         qa = torch.empty((N, self.H * self.D), dtype=q.dtype, device=q.device)
-        ops.head_linear(q, self.dn + self.dr, self.uk_t.weight, qa, self.D)              # Uk_h^T qn_h -> qa[:, h, :R]
-        ops.rope_tail(q, self.dn + self.dr, self.dn, qa, self.D, self.R, self.H, self.dr, ctx.positions, table)
+        # Uk_h^T qn_h -> qa[:, h, :R]; rotate(qr_h) -> qa[:, h, R:R + dr]; zeros behind
+        ops.head_linear(q, self.dn + self.dr, self.uk_t.weight, qa, self.D,
+                        rope_tail=(self.dn, self.R, self.dr, ctx.positions, table))
         a = ops.paged_attention(qa, binding.k_pages, binding.v_pages, group.block_tables, ctx.seg_of_token,
                                 ctx.positions, self.H, 1, self.D, self.scale, 0, batch=ctx)
         out = torch.empty((N, self.H * self.dv), dtype=q.dtype, device=q.device)

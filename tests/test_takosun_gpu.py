@@ -153,6 +153,21 @@ def test_latent_rows_and_rotated_query_parts(dtype, R, dr, rot, D, ps):
     got = qa.float().cpu().reshape(N, H, D)
     close(got[..., R:R + dr], ref, dtype)
     assert (got[..., :R] == 5.0).all() and (got[..., R + dr:] == 0).all()
+    # the same from the launch of the per-head products, which fill the columns before it
+    for n_tok in (N, 3):
+        Wk = (torch.randn((H, R, dn), generator=g) / math.sqrt(dn)).to(dtype)
+        qa = torch.full((n_tok, H * D), 5.0, dtype=dtype).cuda()
+        o.head_linear(q[:n_tok].cuda(), dn + dr, Wk.cuda(), qa, D, rope_tail=(dn, R, dr, pos[:n_tok].cuda(), table.cuda()))
+        got = qa.float().cpu().reshape(n_tok, H, D)
+        close(got[..., R:R + dr], ref[:n_tok], dtype)
+        close(got[..., :R], torch.einsum("nhd,hrd->nhr", qf[:n_tok, :, :dn], Wk.float()), dtype, 2.0)
+        assert (got[..., R + dr:] == 0).all()
+    # the norm of another part of the same rows from the cache write's launch
+    x2 = torch.randn((N, 7 + R + dr), generator=g).to(dtype)
+    w2 = 1 + 0.3 * torch.randn(7, generator=g)
+    got = o.latent_cache_write(x2.cuda()[:, 7:], w.cuda(), 1e-5, R, dr, pos.cuda(), table.cuda(), slots.cuda(), k, v,
+                               also_norm=x2.cuda()[:, :7], also_weight=w2.cuda())
+    close(got, t_rms_norm(x2[:, :7].float(), w2, 1e-5), dtype)
 
 
 @pytest.mark.parametrize("dtype", DTYPES)

@@ -179,7 +179,8 @@ class TorchOps:
         a, b = v[..., :half], v[..., half:rot]
         return torch.cat([a * c - b * s, b * c + a * s, v[..., rot:]], dim=-1)
 
-    def latent_cache_write(self, x, weight, eps, rank, rot_width, positions, table, slots, k_pages, v_pages):
+    def latent_cache_write(self, x, weight, eps, rank, rot_width, positions, table, slots, k_pages, v_pages,
+                           also_norm=None, also_weight=None):
         ps, D = k_pages.shape[2], k_pages.shape[3]
         xf = x.to(torch.float32)
         c = self._gn(xf[:, :rank], weight, 1, eps)
@@ -192,9 +193,15 @@ class TorchOps:
             if s >= 0:
                 k_pages[s // ps, 0, s % ps, :] = row[n]
                 v_pages[s // ps, 0, :, s % ps] = row[n]
+        if also_norm is not None:
+            return self._gn(also_norm.to(torch.float32), also_weight, 1, eps).to(x.dtype)
+        return None
 
-    def head_linear(self, x, x_head, weight, out, out_head, gate=None):
+    def head_linear(self, x, x_head, weight, out, out_head, gate=None, rope_tail=None):
         H, O, K = weight.shape
+        if rope_tail is not None:
+            x_at, out_at, width, positions, table = rope_tail
+            self.rope_tail(x, x_head, x_at, out, out_head, out_at, H, width, positions, table)
         for h in range(H):
             y = x[:, h * x_head:h * x_head + K].to(torch.float32) @ weight[h].to(torch.float32).t()
             if gate is not None:

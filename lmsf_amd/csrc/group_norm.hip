@@ -70,6 +70,7 @@ __global__ __launch_bounds__(GN_MAX_THREADS) void group_norm_kernel(
       const float r = row[i];
       hist[(long)hist_index * hist_stride + (long)n * W + i] = r;
       float x = 0.f;
+#pragma unroll 8
       for (int j = 0; j < hist_index; ++j) x += mix[j] * hist[(long)j * hist_stride + (long)n * W + i];
       x += mix[hist_index] * r;
       row[i] = x;

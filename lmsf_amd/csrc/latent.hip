@@ -223,6 +223,7 @@ __global__ __launch_bounds__(256) void head_linear_mfma_kernel(
   f32x4_t acc[MT];
 #pragma unroll
   for (int mt = 0; mt < MT; ++mt) acc[mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+#pragma unroll 4
   for (int k = 0; k < K; k += 32) {
     const bf16x8_t fa = *reinterpret_cast<const bf16x8_t*>(wa + k);
     bf16x8_t fb[MT];

@@ -163,10 +163,10 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   }
 }
 
-// One tile of pairs against 128 outputs of its expert (32 a wave). GATED: x = the tokens' vectors (row of pair p: p / top),
+// One tile of pairs against 64 * NO outputs of its expert (16 * NO a wave). GATED: x = the tokens' vectors (row of pair p: p / top),
 // Wm = Wgu, K = W, O = F, y = act [P, F] bfloat16 = silu(gate) * up; else x = act (row of pair p: p), Wm = Wd, K = F,
 // O = W, y = float32 rows [P, W].
-template <bool GATED>
+template <bool GATED, int NO>
 __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict__ x, long x_stride, int top,
                                                        const bf16_t* __restrict__ Wm, const int* __restrict__ order,
                                                        const int* __restrict__ tiles, const int* __restrict__ n_tiles,
@@ -176,7 +176,7 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
   const int e = tiles[3 * t], place = tiles[3 * t + 1], count = tiles[3 * t + 2];
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int fr = lane % 16, fg = lane / 16;
-  constexpr int NO = 2;                    // tiles of 16 outputs a wave
+  // NO: tiles of 16 outputs a wave (2 where there are tiles enough to fill the chip, else 1 and twice the workgroups)
   constexpr int NA = GATED ? 2 * NO : NO;  // tiles of rows of W a wave: gate and up rows of the same outputs
   const int o0 = blockIdx.y * (64 * NO) + wave * (16 * NO);
   if (o0 >= O) return;
@@ -199,17 +199,33 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
   for (int a = 0; a < NA; ++a)
 #pragma unroll
     for (int mt = 0; mt < 4; ++mt) acc[a][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  // the next step's operands are asked for before this step's are multiplied. With few tiles (NO == 1) a row of W is
+  // read by one workgroup or two and its loads are non-temporal; with many, the tiles of one expert read it again
+  // and again and it should stay in the caches (2,048 tokens: 498 against 350 us with non-temporal loads)
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+#define MOE_LOAD_W(p) (NO == 1 ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)) : *reinterpret_cast<const u32x4*>(p))
+  u32x4 na[NA], nb[4];
+#pragma unroll
+  for (int a = 0; a < NA; ++a) na[a] = MOE_LOAD_W(wa[a]);
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) nb[mt] = *reinterpret_cast<const u32x4*>(xb[mt]);
   for (int k = 0; k < K; k += 32) {
     bf16x8_t fa[NA], fb[4];
 #pragma unroll
-    for (int a = 0; a < NA; ++a) fa[a] = *reinterpret_cast<const bf16x8_t*>(wa[a] + k);
+    for (int a = 0; a < NA; ++a) fa[a] = *reinterpret_cast<const bf16x8_t*>(&na[a]);
 #pragma unroll
-    for (int mt = 0; mt < 4; ++mt) fb[mt] = *reinterpret_cast<const bf16x8_t*>(xb[mt] + k);
+    for (int mt = 0; mt < 4; ++mt) fb[mt] = *reinterpret_cast<const bf16x8_t*>(&nb[mt]);
+    const int kn = k + 32 < K ? k + 32 : k;
+#pragma unroll
+    for (int a = 0; a < NA; ++a) na[a] = MOE_LOAD_W(wa[a] + kn);
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) nb[mt] = *reinterpret_cast<const u32x4*>(xb[mt] + kn);
 #pragma unroll
     for (int a = 0; a < NA; ++a)
 #pragma unroll
       for (int mt = 0; mt < 4; ++mt) acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[a], fb[mt], acc[a][mt], 0, 0, 0);
   }
+#undef MOE_LOAD_W
   // lane: pair fr of every tile of pairs, outputs o0 + a * 16 + fg * 4 .. + 3
 #pragma unroll
   for (int mt = 0; mt < 4; ++mt) {
@@ -275,11 +291,19 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
     int* n_tiles = tiles + 3 * (max_tiles + 1);
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)3 * E * 4, stream, ids, table, vocab, top, E, P,
                        order, tiles, n_tiles);
-    hipLaunchKernelGGL((moe_tile_kernel<true>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream, (const bf16_t*)h,
-                       h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
-    hipLaunchKernelGGL((moe_tile_kernel<false>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
-                       (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows, W,
-                       F);
+    if ((long)max_tiles * ((F + 127) / 128) >= 512) {
+      hipLaunchKernelGGL((moe_tile_kernel<true, 2>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
+                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
+      hipLaunchKernelGGL((moe_tile_kernel<false, 2>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
+                         (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows,
+                         W, F);
+    } else {
+      hipLaunchKernelGGL((moe_tile_kernel<true, 1>), dim3(max_tiles, (F + 63) / 64), dim3(256), 0, stream,
+                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
+      hipLaunchKernelGGL((moe_tile_kernel<false, 1>), dim3(max_tiles, (W + 63) / 64), dim3(256), 0, stream,
+                         (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows,
+                         W, F);
+    }
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, scratch_rows, top, weight,
                        (const bf16_t*)base, base_stride, (bf16_t*)out, out_stride, W);
     LMSF_LAUNCH_CHECK("table_moe (grouped)");

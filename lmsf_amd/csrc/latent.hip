@@ -273,7 +273,8 @@ extern "C" int lmsf_head_linear(const void* x, int dtype, long x_stride, int x_h
   const bool rows16 = lmsf_aligned16(x) && lmsf_aligned16(W) && (x_stride * es) % 16 == 0 && ((long)x_head * es) % 16 == 0;
   if (dtype == LMSF_BF16 && K % 32 == 0 && rows16) {
     const RopeTailArgs tail = {positions, table, rot, max_pos, x_at, y_at, dr};
-    if (n_tokens <= 32)
+    // tiles of 16 tokens a workgroup: 4 where that still gives workgroups enough to fill the chip, else 1
+    if (n_tokens <= 32 || (long)((n_tokens + 63) / 64) * H * ((O + 63) / 64) < 512)
       hipLaunchKernelGGL(head_linear_mfma_kernel<1>, dim3((n_tokens + 15) / 16, H, (O + 63) / 64), dim3(256), 0, stream,
                          (const bf16_t*)x, x_stride, x_head, (const bf16_t*)W, (bf16_t*)y, y_stride, y_head,
                          (const bf16_t*)gate, gate_stride, n_tokens, O, K, tail);

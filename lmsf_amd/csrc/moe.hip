@@ -126,10 +126,12 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
 #define MOE_TILE 64          // pairs a tile holds (four matrix-core tiles of 16)
 
 // Groups the P = N * top pairs by expert. order[i]: the pair at place i of the grouped sequence; tiles: for every
-// tile its expert, its first place and its number of pairs; n_tiles[0]: how many tiles there are. One workgroup.
+// tile (of up to ``tile_pairs`` pairs) its expert, its first place and its number of pairs; n_tiles[0]: how many
+// tiles there are. One workgroup.
 __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__ ids, const int* __restrict__ table,
-                                                        int vocab, int top, int E, int P, int* __restrict__ order,
-                                                        int* __restrict__ tiles, int* __restrict__ n_tiles) {
+                                                        int vocab, int top, int E, int P, int tile_pairs,
+                                                        int* __restrict__ order, int* __restrict__ tiles,
+                                                        int* __restrict__ n_tiles) {
   extern __shared__ int sm[];   // [E] counts, [E] first places, [E] fill counters
   int* cnt = sm;
   int* first = sm + E;
@@ -145,10 +147,10 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
     int at = 0, t = 0;
     for (int e = 0; e < E; ++e) {
       first[e] = at;
-      for (int s = 0; s < cnt[e]; s += MOE_TILE) {
+      for (int s = 0; s < cnt[e]; s += tile_pairs) {
         tiles[3 * t] = e;
         tiles[3 * t + 1] = at + s;
-        tiles[3 * t + 2] = min(MOE_TILE, cnt[e] - s);
+        tiles[3 * t + 2] = min(tile_pairs, cnt[e] - s);
         ++t;
       }
       at += cnt[e];
@@ -176,7 +178,8 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
   const int e = tiles[3 * t], place = tiles[3 * t + 1], count = tiles[3 * t + 2];
   const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
   const int fr = lane % 16, fg = lane / 16;
-  // NO: tiles of 16 outputs a wave (2 where there are tiles enough to fill the chip, else 1 and twice the workgroups)
+  // NO: tiles of 16 outputs a wave: as many that a wave holds four tiles of rows of W against its four tiles of pairs
+  // (2 in the gated product, 4 in the other) where there are tiles enough to fill the chip, else 1 and more workgroups
   constexpr int NA = GATED ? 2 * NO : NO;  // tiles of rows of W a wave: gate and up rows of the same outputs
   const int o0 = blockIdx.y * (64 * NO) + wave * (16 * NO);
   if (o0 >= O) return;
@@ -246,6 +249,117 @@ __global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict_
   }
 }
 
+// The same tile product for many pairs an expert: tiles of 128 pairs against 128 outputs, operands through LDS. A step
+// of 32 k: the workgroup copies the rows of W (128, or 128 gate + 128 up) and the 128 pairs' rows, 64 bytes of each, into
+// LDS with 16-byte loads (the next step's while this step is multiplied: two buffers, one barrier a step), and every
+// wave of the 2 x 2 reads the fragments of its 64 pairs and 64 outputs from there (rows of 64 bytes back to back: a
+// fragment's 64 lanes read 1 KB in a row, no bank conflicts). Per byte that comes from memory 2.7 times the
+// multiplications of the form above, whose waves each fetch their operands themselves.
+#define MOE_BIG_TILE 128
+
+template <bool GATED>
+__global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restrict__ x, long x_stride, int top,
+                                                           const bf16_t* __restrict__ Wm, const int* __restrict__ order,
+                                                           const int* __restrict__ tiles, const int* __restrict__ n_tiles,
+                                                           void* __restrict__ y, int O, int K) {
+  constexpr int AR = GATED ? 256 : 128;            // rows of W a step
+  constexpr int NLA = AR * 4 / 256;                // 16-byte pieces of W a thread copies a step
+  constexpr int NLB = MOE_BIG_TILE * 4 / 256;      // and of the pairs' rows
+  constexpr int NA = GATED ? 8 : 4;                // fragments of W a wave
+  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][(AR + MOE_BIG_TILE) * 64];
+  const int t = blockIdx.x;
+  if (t >= n_tiles[0]) return;
+  const int e = tiles[3 * t], place = tiles[3 * t + 1], count = tiles[3 * t + 2];
+  const int tid = threadIdx.x, wave = tid / LMSF_WAVE, lane = tid % LMSF_WAVE;
+  const int fr = lane % 16, fg = lane / 16;
+  const int wr = wave / 2, wc = wave % 2;          // the wave's 64 pairs and 64 outputs
+  const int o_base = blockIdx.y * 128;
+  // what this thread copies: piece (tid % 4) of rows tid / 4, + 64, ...
+  const bf16_t* ga[NLA];
+  const bf16_t* gb[NLB];
+#pragma unroll
+  for (int i = 0; i < NLA; ++i) {
+    const int r = tid / 4 + i * 64;                // 0 .. AR-1; gated: rows 128 .. 255 are the up rows
+    const int o = min(o_base + (r & 127), O - 1);
+    ga[i] = Wm + ((long)e * (GATED ? 2 : 1) * O + (GATED && r >= 128 ? O : 0) + o) * K + (tid % 4) * 8;
+  }
+#pragma unroll
+  for (int i = 0; i < NLB; ++i) {
+    const int p = order[place + min(tid / 4 + i * 64, count - 1)];
+    gb[i] = x + (long)(GATED ? p / top : p) * x_stride + (tid % 4) * 8;
+  }
+  f32x4_t acc[NA][4];
+#pragma unroll
+  for (int a = 0; a < NA; ++a)
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt) acc[a][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
+  u32x4 ra[NLA], rb[NLB];
+#pragma unroll
+  for (int i = 0; i < NLA; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ga[i]);
+#pragma unroll
+  for (int i = 0; i < NLB; ++i) rb[i] = *reinterpret_cast<const u32x4*>(gb[i]);
+#pragma unroll
+  for (int i = 0; i < NLA; ++i) *reinterpret_cast<u32x4*>(lds[0] + (tid / 4 + i * 64) * 64 + (tid % 4) * 16) = ra[i];
+#pragma unroll
+  for (int i = 0; i < NLB; ++i) *reinterpret_cast<u32x4*>(lds[0] + (AR + tid / 4 + i * 64) * 64 + (tid % 4) * 16) = rb[i];
+  __syncthreads();
+  int cur = 0;
+  for (int k = 0; k < K; k += 32) {
+    const bool more = k + 32 < K;
+    if (more) {
+#pragma unroll
+      for (int i = 0; i < NLA; ++i) ra[i] = *reinterpret_cast<const u32x4*>(ga[i] + k + 32);
+#pragma unroll
+      for (int i = 0; i < NLB; ++i) rb[i] = *reinterpret_cast<const u32x4*>(gb[i] + k + 32);
+    }
+    const unsigned char* buf = lds[cur];
+    bf16x8_t fa[NA], fb[4];
+#pragma unroll
+    for (int a = 0; a < NA; ++a) {
+      // fragment a: outputs wc * 64 + (a % 4) * 16 ..; gated: a >= 4 are the up rows of the same outputs
+      const int row = (GATED && a >= 4 ? 128 : 0) + wc * 64 + (a & 3) * 16 + fr;
+      fa[a] = *reinterpret_cast<const bf16x8_t*>(buf + row * 64 + fg * 16);
+    }
+#pragma unroll
+    for (int mt = 0; mt < 4; ++mt)
+      fb[mt] = *reinterpret_cast<const bf16x8_t*>(buf + (AR + wr * 64 + mt * 16 + fr) * 64 + fg * 16);
+#pragma unroll
+    for (int a = 0; a < NA; ++a)
+#pragma unroll
+      for (int mt = 0; mt < 4; ++mt) acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[a], fb[mt], acc[a][mt], 0, 0, 0);
+    if (more) {
+      unsigned char* nxt = lds[cur ^ 1];
+#pragma unroll
+      for (int i = 0; i < NLA; ++i) *reinterpret_cast<u32x4*>(nxt + (tid / 4 + i * 64) * 64 + (tid % 4) * 16) = ra[i];
+#pragma unroll
+      for (int i = 0; i < NLB; ++i) *reinterpret_cast<u32x4*>(nxt + (AR + tid / 4 + i * 64) * 64 + (tid % 4) * 16) = rb[i];
+    }
+    __syncthreads();
+    cur ^= 1;
+  }
+  // lane: pair wr * 64 + mt * 16 + fr, outputs o_base + wc * 64 + a * 16 + fg * 4 .. + 3
+#pragma unroll
+  for (int mt = 0; mt < 4; ++mt) {
+    const int slot = wr * 64 + mt * 16 + fr;
+    if (slot >= count) continue;
+    const int p = order[place + slot];
+#pragma unroll
+    for (int a = 0; a < 4; ++a)
+#pragma unroll
+      for (int j = 0; j < 4; ++j) {
+        const int o = o_base + wc * 64 + a * 16 + fg * 4 + j;
+        if (o >= O) continue;
+        if (GATED) {
+          const float g = bf16_to_f32(f32_to_bf16(acc[a][mt][j])), u = bf16_to_f32(f32_to_bf16(acc[NA - 4 + a][mt][j]));
+          reinterpret_cast<bf16_t*>(y)[(long)p * O + o] = f32_to_bf16(g / (1.f + expf(-g)) * u);
+        } else {
+          reinterpret_cast<float*>(y)[(long)p * O + o] = acc[a][mt][j];
+        }
+      }
+  }
+}
+
 // out[n, o] = base[n, o] + weight * sum_k rows[n * top + k, o]
 __global__ __launch_bounds__(256) void moe_combine_kernel(const float* __restrict__ rows, int top, float weight,
                                                           const bf16_t* __restrict__ base, long base_stride,
@@ -285,16 +399,25 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
   if (n_tokens <= 0) return 0;
   if (lmsf_table_moe_grouped(dtype, n_tokens, top, E, F, W, h_stride) && scratch_ints && scratch_rows &&
       lmsf_aligned16(h) && lmsf_aligned16(Wgu) && lmsf_aligned16(Wd) && lmsf_aligned16(act)) {
-    const int P = n_tokens * top, max_tiles = P / MOE_TILE + E;
+    // many pairs an expert: tiles of 128 through LDS; else tiles of 64 with operands straight from memory
+    const int P = n_tokens * top;
+    const bool big = P / E >= 96;
+    const int tile_pairs = big ? MOE_BIG_TILE : MOE_TILE, max_tiles = P / tile_pairs + E;
     int* order = scratch_ints;
     int* tiles = order + P;
-    int* n_tiles = tiles + 3 * (max_tiles + 1);
+    int* n_tiles = tiles + 3 * (P / MOE_TILE + E + 1);
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)3 * E * 4, stream, ids, table, vocab, top, E, P,
-                       order, tiles, n_tiles);
-    if ((long)max_tiles * ((F + 127) / 128) >= 512) {
+                       tile_pairs, order, tiles, n_tiles);
+    if (big) {
+      hipLaunchKernelGGL((moe_tile_lds_kernel<true>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
+                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
+      hipLaunchKernelGGL((moe_tile_lds_kernel<false>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
+                         (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows,
+                         W, F);
+    } else if ((long)max_tiles * ((F + 127) / 128) >= 512) {
       hipLaunchKernelGGL((moe_tile_kernel<true, 2>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
                          (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
-      hipLaunchKernelGGL((moe_tile_kernel<false, 2>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
+      hipLaunchKernelGGL((moe_tile_kernel<false, 4>), dim3(max_tiles, (W + 255) / 256), dim3(256), 0, stream,
                          (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows,
                          W, F);
     } else {

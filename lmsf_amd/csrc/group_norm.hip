@@ -14,7 +14,8 @@
 //   out[row] = wn ? gn(x; wn) : x                           the norm *before* the next sublayer
 //
 // All arithmetic is float32; branch and out are float32 or bfloat16, the weights float32. One workgroup a row
-// (256 to 1,024 threads), the row kept in LDS between the passes.
+// (256 to 1,024 threads), the row kept in LDS between the passes; the stream's row and the earlier results are asked
+// for before the first pass, so that the passes do not each wait for memory.
 #include "common.h"
 
 #include <math.h>
@@ -48,19 +49,32 @@ __global__ __launch_bounds__(GN_MAX_THREADS) void group_norm_kernel(
     float* __restrict__ hist, long hist_stride, int hist_index, const float* __restrict__ mix,
     const float* __restrict__ wn, TO* __restrict__ out, long out_stride, const int* __restrict__ rows, int W,
     int groups, float eps_b, float eps_n) {
-  extern __shared__ float row[];   // [W]
+  extern __shared__ float row[];   // [W] the row; [W] the stream's row; [W] the earlier results' share of the average
+  float* res = row + W;
+  float* before = row + 2 * W;
   __shared__ float red[16];
   const int n = blockIdx.x;
   const int src = rows ? rows[n] : n;
+  // everything that comes from memory is asked for at once: the passes below would otherwise each wait for their own
+  if (residual)
+    for (int i = threadIdx.x; i < W; i += GN_THREADS) res[i] = residual[(long)src * W + i];
+  if (hist)
+    for (int i = threadIdx.x; i < W; i += GN_THREADS) {
+      float x = 0.f;
+#pragma unroll 8
+      for (int j = 0; j < hist_index; ++j) x += mix[j] * hist[(long)j * hist_stride + (long)n * W + i];
+      before[i] = x;
+    }
   if (branch) {
     for (int i = threadIdx.x; i < W; i += GN_THREADS) row[i] = to_f32<TB>(branch[(long)n * branch_stride + i]);
     __syncthreads();
     gn_normalize(row, wb, W, groups, eps_b, red);
   }
+  // (each thread reads back the entries of res and before that it wrote itself)
   if (residual) {
     const bool store = branch && !rows && !hist;
     for (int i = threadIdx.x; i < W; i += GN_THREADS) {
-      const float r = residual[(long)src * W + i] + (branch ? row[i] : 0.f);
+      const float r = res[i] + (branch ? row[i] : 0.f);
       row[i] = r;
       if (store) residual[(long)n * W + i] = r;
     }
@@ -69,10 +83,7 @@ __global__ __launch_bounds__(GN_MAX_THREADS) void group_norm_kernel(
     for (int i = threadIdx.x; i < W; i += GN_THREADS) {
       const float r = row[i];
       hist[(long)hist_index * hist_stride + (long)n * W + i] = r;
-      float x = 0.f;
-#pragma unroll 8
-      for (int j = 0; j < hist_index; ++j) x += mix[j] * hist[(long)j * hist_stride + (long)n * W + i];
-      x += mix[hist_index] * r;
+      const float x = before[i] + mix[hist_index] * r;
       row[i] = x;
       residual[(long)n * W + i] = x;
     }
@@ -103,7 +114,7 @@ extern "C" int lmsf_group_norm(const void* branch, int branch_dtype, long branch
                                int n_rows, int W, int groups, float eps_b, float eps_n, hipStream_t stream) {
   LMSF_CHECK(branch || residual, "group_norm: neither a branch nor a residual");
   LMSF_CHECK(W > 0 && groups > 0 && W % groups == 0, "group_norm: %d columns do not split into %d groups", W, groups);
-  LMSF_CHECK((size_t)W * 4 <= 160 * 1024 - 256, "group_norm: a row of %d columns does not fit LDS", W);
+  LMSF_CHECK((size_t)W * 12 <= 160 * 1024 - 256, "group_norm: three rows of %d columns do not fit LDS", W);
   LMSF_CHECK(!branch || wb, "group_norm: a branch needs its weight");
   LMSF_CHECK(!branch || branch_stride >= W, "group_norm: branch rows overlap");
   LMSF_CHECK(!out || out_stride >= W, "group_norm: output rows overlap");
@@ -112,7 +123,7 @@ extern "C" int lmsf_group_norm(const void* branch, int branch_dtype, long branch
   LMSF_CHECK(branch_dtype == LMSF_F32 || branch_dtype == LMSF_BF16, "group_norm: unknown dtype code %d", branch_dtype);
   LMSF_CHECK(out_dtype == LMSF_F32 || out_dtype == LMSF_BF16, "group_norm: unknown dtype code %d", out_dtype);
   if (n_rows <= 0) return 0;
-  const size_t smem = (size_t)W * 4;
+  const size_t smem = (size_t)W * 12;
   if (smem > 64 * 1024) {
     // (once per instantiation would do; the call is cheap)
     hipFuncSetAttribute((const void*)group_norm_kernel<float, float>, hipFuncAttributeMaxDynamicSharedMemorySize, (int)smem);

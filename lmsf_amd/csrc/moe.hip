@@ -7,10 +7,9 @@
 // Few tokens (decoding), and float32 at any number: every (token, choice) streams its expert's rows, a wave per
 // output, the token's vector in LDS, 16-byte loads where the rows allow them.
 // Many tokens in bfloat16: the (token, choice) pairs are grouped by expert on the device (one small kernel: counts,
-// offsets, an order, a list of tiles of up to 64 pairs of one expert), and each tile runs on the matrix cores
-// against a block of its expert's rows: A = 16 rows of W x 32 k, B = 16 pairs x 32 k, four tiles of pairs and, in the
-// gated product, the gate and the up rows of the same 16 outputs a wave, operands straight from memory. The down
-// product leaves float32 rows per pair; a last kernel adds a token's pairs and the shared part. A pair's result
+// offsets, an order, a list of tiles of up to 128 pairs of one expert), and each tile runs on the matrix cores
+// against 128 of its expert's outputs (A = 16 rows of W x 32 k, B = 16 pairs x 32 k; in the gated product the gate
+// and the up rows of the same outputs), operands through LDS. The down product leaves float32 rows per pair; a last kernel adds a token's pairs and the shared part. A pair's result
 // does not depend on where in its tile it lies, so the order inside an expert's group (atomic counters) is free.
 // Accumulation in float32 throughout.
 #include "common.h"
@@ -123,7 +122,7 @@ __global__ __launch_bounds__(MOE_THREADS) void moe_down_kernel(
 
 // ---------------------------------------------------------------- many tokens: grouped by expert, matrix cores
 
-#define MOE_TILE 64          // pairs a tile holds (four matrix-core tiles of 16)
+#define MOE_TILE 128         // pairs a tile holds
 
 // Groups the P = N * top pairs by expert. order[i]: the pair at place i of the grouped sequence; tiles: for every
 // tile (of up to ``tile_pairs`` pairs) its expert, its first place and its number of pairs; n_tiles[0]: how many
@@ -165,97 +164,15 @@ __global__ __launch_bounds__(1024) void moe_group_kernel(const int* __restrict__
   }
 }
 
-// One tile of pairs against 64 * NO outputs of its expert (16 * NO a wave). GATED: x = the tokens' vectors (row of pair p: p / top),
-// Wm = Wgu, K = W, O = F, y = act [P, F] bfloat16 = silu(gate) * up; else x = act (row of pair p: p), Wm = Wd, K = F,
-// O = W, y = float32 rows [P, W].
-template <bool GATED, int NO>
-__global__ __launch_bounds__(256) void moe_tile_kernel(const bf16_t* __restrict__ x, long x_stride, int top,
-                                                       const bf16_t* __restrict__ Wm, const int* __restrict__ order,
-                                                       const int* __restrict__ tiles, const int* __restrict__ n_tiles,
-                                                       void* __restrict__ y, int O, int K) {
-  const int t = blockIdx.x;
-  if (t >= n_tiles[0]) return;
-  const int e = tiles[3 * t], place = tiles[3 * t + 1], count = tiles[3 * t + 2];
-  const int wave = threadIdx.x / LMSF_WAVE, lane = threadIdx.x % LMSF_WAVE;
-  const int fr = lane % 16, fg = lane / 16;
-  // NO: tiles of 16 outputs a wave: as many that a wave holds four tiles of rows of W against its four tiles of pairs
-  // (2 in the gated product, 4 in the other) where there are tiles enough to fill the chip, else 1 and more workgroups
-  constexpr int NA = GATED ? 2 * NO : NO;  // tiles of rows of W a wave: gate and up rows of the same outputs
-  const int o0 = blockIdx.y * (64 * NO) + wave * (16 * NO);
-  if (o0 >= O) return;
-  const bf16_t* wa[NA];
-#pragma unroll
-  for (int a = 0; a < NO; ++a) {
-    const int orow = min(o0 + a * 16 + fr, O - 1);
-    wa[a] = Wm + ((long)e * (GATED ? 2 : 1) * O + orow) * K + fg * 8;
-    if (GATED) wa[NO + a] = Wm + ((long)e * 2 * O + O + orow) * K + fg * 8;
-  }
-  const bf16_t* xb[4];
-  int pair[4];
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    pair[mt] = order[place + min(mt * 16 + fr, count - 1)];
-    xb[mt] = x + (long)(GATED ? pair[mt] / top : pair[mt]) * x_stride + fg * 8;
-  }
-  f32x4_t acc[NA][4];
-#pragma unroll
-  for (int a = 0; a < NA; ++a)
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) acc[a][mt] = f32x4_t{0.f, 0.f, 0.f, 0.f};
-  // the next step's operands are asked for before this step's are multiplied. With few tiles (NO == 1) a row of W is
-  // read by one workgroup or two and its loads are non-temporal; with many, the tiles of one expert read it again
-  // and again and it should stay in the caches (2,048 tokens: 498 against 350 us with non-temporal loads)
-  typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-#define MOE_LOAD_W(p) (NO == 1 ? __builtin_nontemporal_load(reinterpret_cast<const u32x4*>(p)) : *reinterpret_cast<const u32x4*>(p))
-  u32x4 na[NA], nb[4];
-#pragma unroll
-  for (int a = 0; a < NA; ++a) na[a] = MOE_LOAD_W(wa[a]);
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) nb[mt] = *reinterpret_cast<const u32x4*>(xb[mt]);
-  for (int k = 0; k < K; k += 32) {
-    bf16x8_t fa[NA], fb[4];
-#pragma unroll
-    for (int a = 0; a < NA; ++a) fa[a] = *reinterpret_cast<const bf16x8_t*>(&na[a]);
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) fb[mt] = *reinterpret_cast<const bf16x8_t*>(&nb[mt]);
-    const int kn = k + 32 < K ? k + 32 : k;
-#pragma unroll
-    for (int a = 0; a < NA; ++a) na[a] = MOE_LOAD_W(wa[a] + kn);
-#pragma unroll
-    for (int mt = 0; mt < 4; ++mt) nb[mt] = *reinterpret_cast<const u32x4*>(xb[mt] + kn);
-#pragma unroll
-    for (int a = 0; a < NA; ++a)
-#pragma unroll
-      for (int mt = 0; mt < 4; ++mt) acc[a][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(fa[a], fb[mt], acc[a][mt], 0, 0, 0);
-  }
-#undef MOE_LOAD_W
-  // lane: pair fr of every tile of pairs, outputs o0 + a * 16 + fg * 4 .. + 3
-#pragma unroll
-  for (int mt = 0; mt < 4; ++mt) {
-    if (mt * 16 + fr >= count) continue;
-#pragma unroll
-    for (int a = 0; a < NO; ++a)
-#pragma unroll
-      for (int j = 0; j < 4; ++j) {
-        const int o = o0 + a * 16 + fg * 4 + j;
-        if (o >= O) continue;
-        if (GATED) {
-          const float g = bf16_to_f32(f32_to_bf16(acc[a][mt][j])), u = bf16_to_f32(f32_to_bf16(acc[NA - NO + a][mt][j]));
-          reinterpret_cast<bf16_t*>(y)[(long)pair[mt] * O + o] = f32_to_bf16(g / (1.f + expf(-g)) * u);
-        } else {
-          reinterpret_cast<float*>(y)[(long)pair[mt] * O + o] = acc[a][mt][j];
-        }
-      }
-  }
-}
-
-// The same tile product for many pairs an expert: tiles of 128 pairs against 128 outputs, operands through LDS. A step
-// of 32 k: the workgroup copies the rows of W (128, or 128 gate + 128 up) and the 128 pairs' rows, 64 bytes of each, into
+// One tile of up to 128 pairs against 128 outputs of its expert, operands through LDS. GATED: x = the tokens' vectors
+// (row of pair p: p / top), Wm = Wgu, K = W, O = F, y = act [P, F] bfloat16 = silu(gate) * up; else x = act (row of pair
+// p: p), Wm = Wd, K = F, O = W, y = float32 rows [P, W]. A step of 32 k: the workgroup copies the rows of W (128, or 128 gate + 128 up) and the 128 pairs' rows, 64 bytes of each, into
 // LDS with 16-byte loads (the next step's while this step is multiplied: two buffers, one barrier a step), and every
 // wave of the 2 x 2 reads the fragments of its 64 pairs and 64 outputs from there (rows of 64 bytes back to back: a
-// fragment's 64 lanes read 1 KB in a row, no bank conflicts). Per byte that comes from memory 2.7 times the
-// multiplications of the form above, whose waves each fetch their operands themselves.
-#define MOE_BIG_TILE 128
+// fragment's 64 lanes read 1 KB in a row, no bank conflicts). A first form whose waves fetched their fragments
+// themselves, straight from memory in tiles of 64 pairs, did 2.7 times fewer multiplications per byte fetched and lost
+// at every number of pairs: 2,048 tokens (256 pairs an expert) 319 against 194 us for the four kernels, 512 tokens 230
+// against 98, 64 tokens (8 pairs an expert, every tile mostly empty) 101 against 83.
 
 template <bool GATED>
 __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restrict__ x, long x_stride, int top,
@@ -264,10 +181,10 @@ __global__ __launch_bounds__(256) void moe_tile_lds_kernel(const bf16_t* __restr
                                                            void* __restrict__ y, int O, int K) {
   constexpr int AR = GATED ? 256 : 128;            // rows of W a step
   constexpr int NLA = AR * 4 / 256;                // 16-byte pieces of W a thread copies a step
-  constexpr int NLB = MOE_BIG_TILE * 4 / 256;      // and of the pairs' rows
+  constexpr int NLB = MOE_TILE * 4 / 256;      // and of the pairs' rows
   constexpr int NA = GATED ? 8 : 4;                // fragments of W a wave
   typedef unsigned int u32x4 __attribute__((ext_vector_type(4)));
-  __shared__ __attribute__((aligned(16))) unsigned char lds[2][(AR + MOE_BIG_TILE) * 64];
+  __shared__ __attribute__((aligned(16))) unsigned char lds[2][(AR + MOE_TILE) * 64];
   const int t = blockIdx.x;
   if (t >= n_tiles[0]) return;
   const int e = tiles[3 * t], place = tiles[3 * t + 1], count = tiles[3 * t + 2];
@@ -399,34 +316,17 @@ extern "C" int lmsf_table_moe(const void* h, int dtype, long h_stride, const voi
   if (n_tokens <= 0) return 0;
   if (lmsf_table_moe_grouped(dtype, n_tokens, top, E, F, W, h_stride) && scratch_ints && scratch_rows &&
       lmsf_aligned16(h) && lmsf_aligned16(Wgu) && lmsf_aligned16(Wd) && lmsf_aligned16(act)) {
-    // many pairs an expert: tiles of 128 through LDS; else tiles of 64 with operands straight from memory
-    const int P = n_tokens * top;
-    const bool big = P / E >= 96;
-    const int tile_pairs = big ? MOE_BIG_TILE : MOE_TILE, max_tiles = P / tile_pairs + E;
+    const int P = n_tokens * top, max_tiles = P / MOE_TILE + E;
     int* order = scratch_ints;
     int* tiles = order + P;
-    int* n_tiles = tiles + 3 * (P / MOE_TILE + E + 1);
+    int* n_tiles = tiles + 3 * (max_tiles + 1);
     hipLaunchKernelGGL(moe_group_kernel, dim3(1), dim3(1024), (size_t)3 * E * 4, stream, ids, table, vocab, top, E, P,
-                       tile_pairs, order, tiles, n_tiles);
-    if (big) {
-      hipLaunchKernelGGL((moe_tile_lds_kernel<true>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
-                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
-      hipLaunchKernelGGL((moe_tile_lds_kernel<false>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
-                         (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows,
-                         W, F);
-    } else if ((long)max_tiles * ((F + 127) / 128) >= 512) {
-      hipLaunchKernelGGL((moe_tile_kernel<true, 2>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
-                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
-      hipLaunchKernelGGL((moe_tile_kernel<false, 4>), dim3(max_tiles, (W + 255) / 256), dim3(256), 0, stream,
-                         (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows,
-                         W, F);
-    } else {
-      hipLaunchKernelGGL((moe_tile_kernel<true, 1>), dim3(max_tiles, (F + 63) / 64), dim3(256), 0, stream,
-                         (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
-      hipLaunchKernelGGL((moe_tile_kernel<false, 1>), dim3(max_tiles, (W + 63) / 64), dim3(256), 0, stream,
-                         (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows,
-                         W, F);
-    }
+                       MOE_TILE, order, tiles, n_tiles);
+    hipLaunchKernelGGL((moe_tile_lds_kernel<true>), dim3(max_tiles, (F + 127) / 128), dim3(256), 0, stream,
+                       (const bf16_t*)h, h_stride, top, (const bf16_t*)Wgu, order, tiles, n_tiles, act, F, W);
+    hipLaunchKernelGGL((moe_tile_lds_kernel<false>), dim3(max_tiles, (W + 127) / 128), dim3(256), 0, stream,
+                       (const bf16_t*)act, (long)F, top, (const bf16_t*)Wd, order, tiles, n_tiles, (void*)scratch_rows, W,
+                       F);
     hipLaunchKernelGGL(moe_combine_kernel, dim3(n_tokens), dim3(256), 0, stream, scratch_rows, top, weight,
                        (const bf16_t*)base, base_stride, (bf16_t*)out, out_stride, W);
     LMSF_LAUNCH_CHECK("table_moe (grouped)");

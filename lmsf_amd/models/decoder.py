@@ -45,6 +45,13 @@ class DecoderModel:
                                                                                           b.value_dim):
                     raise ValueError("schedule entry %d cannot read the cache of entry %d: cache shapes differ"
                                      % (i, e.cache_from))
+        # a block that is always followed by the same block is told so (it may then do part of that block's work)
+        followers = {}
+        for e, nxt in zip(self.schedule, self.schedule[1:]):
+            followers.setdefault(e.layer, set()).add(nxt.layer)
+        for li, b in enumerate(self.blocks):
+            if hasattr(b, "link_next") and len(followers.get(li, ())) == 1 and li != self.schedule[-1].layer:   # (the last run is followed by the final norm)
+                b.link_next(self.blocks[next(iter(followers[li]))])
         self.bindings: List[CacheBinding] = [CacheBinding() for _ in self.schedule]
         # a block may return an unfinished product where everything that ever receives it can take one
         takes = [self.blocks[e.layer].accepts_pending_branch for e in self.schedule[1:]] + [self.final_norm.accepts_pending]

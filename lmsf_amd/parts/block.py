@@ -56,7 +56,8 @@ class SandwichDepthBlock(Block):
     averaging. The stream and every X_j are float32. The results lie in one buffer [depth_total + 1, N, W] that
     the first block of a step allocates and the others find in ``ctx.aux``. The addition after the mixer and the
     norm before the feed-forward are one kernel; so are the addition after the feed-forward, the storing of
-    X_k and the averaging. Nothing is left to add when the block returns.
+    X_k, the averaging and (where the model has linked the blocks) the first norm of the block that follows.
+    Nothing is left to add when the block returns.
 
     The reference's only arrangement is the pre-norm one above (core/src/model_executor/models/llama/llama.rs:286-340).
     """
@@ -77,6 +78,13 @@ class SandwichDepthBlock(Block):
             raise ValueError("block %s needs the norms pre_ffn and post_ffn around its feed-forward" % prefix)
         self.mix = build_part("norm", mix, prefix, rt) if mix is not None else None
         self._ffn_takes_ids = bool(getattr(feed_forward, "needs_token_ids", False))
+        self.next_norm = None       # the norm that the block after this one begins with, where the model has linked it
+
+    def link_next(self, following: Block) -> None:
+        """The model tells a block which block always runs after it: this one's last kernel then also computes that
+        one's first norm (one launch a layer less) and leaves it in ``ctx.aux["prenormed"]``."""
+        if isinstance(following, SandwichDepthBlock):
+            self.next_norm = following.norms["pre_mixer"]
 
     def children(self):
         return super().children() + ([self.mix] if self.mix is not None else [])
@@ -92,19 +100,23 @@ class SandwichDepthBlock(Block):
             hist[0].copy_(residual)
             ctx.aux["depth_history"] = hist
         mix = self.mix.weight if self.mix is not None else None
-        h = n["pre_mixer"].forward(residual)
+        h = ctx.aux.pop("prenormed", None)
+        if h is None:
+            h = n["pre_mixer"].forward(residual)
         a = self.mixer.forward(h, ctx, binding)
         if not self.has_ffn:
-            self._close(n["post_mixer"], a, residual, hist, mix)
+            self._close(n["post_mixer"], a, residual, hist, mix, ctx)
             return None
         h = n["post_mixer"].add_normed(a, residual, then=n["pre_ffn"])
         f = self.feed_forward.forward(h, token_ids=ctx.token_ids) if self._ffn_takes_ids else self.feed_forward.forward(h)
-        self._close(n["post_ffn"], f, residual, hist, mix)
+        self._close(n["post_ffn"], f, residual, hist, mix, ctx)
         return None
 
-    def _close(self, norm, branch, residual, hist, mix) -> None:
+    def _close(self, norm, branch, residual, hist, mix, ctx) -> None:
         if mix is None:
-            norm.add_normed(branch, residual)
+            ahead = norm.add_normed(branch, residual, then=self.next_norm)
             hist[self.depth].copy_(residual)
         else:
-            norm.add_normed(branch, residual, history=hist, index=self.depth, mix=mix)
+            ahead = norm.add_normed(branch, residual, then=self.next_norm, history=hist, index=self.depth, mix=mix)
+        if ahead is not None:
+            ctx.aux["prenormed"] = ahead

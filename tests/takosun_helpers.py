@@ -53,6 +53,12 @@ CONFIGS = {
         layer(mixer(3, 12, 20, 6, 300, 20), moe(10, 3, 2, shared=50)),
         layer(mixer(2, 4, 20, 28, 300, 44, kv_from=0), dense(52)),
     ]},
+    # M: sizes at which the matrix-core forms of the per-head products and of the grouped experts run, the cached row
+    # as wide as the matrix-core attention takes (224 + 32), products of many rows and columns
+    "M": {"architecture": "Takosun", "vocab": 300, "width": 1024, "norm": {"eps": 1e-5, "groups": 2}, "layers": [
+        layer(mixer(8, 64, 32, 96, 224, 384, base=50000.0), dense(2048)),
+        layer(mixer(8, 64, 32, 96, 224, 384, base=50000.0, kv_from=0), moe(512, 4, 2, shared=512)),
+    ]},
     "R": {"architecture": "Takosun", "vocab": 50, "width": 32, "norm": {"eps": 1e-5, "groups": 2}, "layers": [
         layer(mixer(1, 32, 4, 16, 12, 8), moe(16, 2, 1, shared=8)),
         layer(mixer(1, 32, 4, 16, 12, 8, kv_from=0), dense(64)),

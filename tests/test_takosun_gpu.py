@@ -213,7 +213,7 @@ def tokens(n, vocab, seed):
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
-@pytest.mark.parametrize("which", sorted(CONFIGS))
+@pytest.mark.parametrize("which", sorted(k for k in CONFIGS if k != "M"))
 def test_four_ways_of_cutting_give_the_plain_logits(tmp_path, which, dtype):
     from lmsf_amd.engine import StepEntry
     core, cfg, w = build(tmp_path, which, dtype)
@@ -240,6 +240,21 @@ def test_four_ways_of_cutting_give_the_plain_logits(tmp_path, which, dtype):
         check(got[k], ref[k], dtype, cfg, w, t, (k, "mixed"))
     core.storage.manager.check_invariants()
     assert core.storage.manager.num_free_pages(0) == 48
+
+
+@pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
+def test_sizes_at_which_the_matrix_core_forms_run(tmp_path, dtype):
+    """Width 1,024: per-head products and grouped experts on the matrix cores, the 17-and-more-rows and many-rows
+    products, attention over a cached row of 256 entries; a prompt in two portions, a second request beside it, then
+    single tokens of both."""
+    from lmsf_amd.engine import StepEntry
+    core, cfg, w = build(tmp_path, "M", dtype, pages=40)
+    V = cfg["vocab"]
+    a, b = tokens(330, V, 21), tokens(70, V, 22)
+    steps = [[("a", 280)], [("a", 40), ("b", 60)]] + [[("a", 1), ("b", 1)]] * 10
+    got = replay(core.executor, StepEntry, {"a": a, "b": b}, steps)
+    for k, t in (("a", a), ("b", b)):
+        check(got[k], plain_logits(cfg, w, t), dtype, cfg, w, t, k)
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

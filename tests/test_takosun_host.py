@@ -35,7 +35,7 @@ def test_the_architecture_is_found_by_its_name():
     assert resolve_architecture({"architecture": "Takosun"}).name == "Takosun"
 
 
-@pytest.mark.parametrize("which", sorted(CONFIGS))
+@pytest.mark.parametrize("which", sorted(k for k in CONFIGS if k != "M"))   # (M: sizes for the GPU kernels)
 def test_whole_prompt(tmp_path, which):
     core, cfg, w = build(tmp_path, which)
     toks = tokens(45, cfg["vocab"], 1)
@@ -43,7 +43,7 @@ def test_whole_prompt(tmp_path, which):
     assert rel_err(out, plain_logits(cfg, w, toks)) < TOL
 
 
-@pytest.mark.parametrize("which", sorted(CONFIGS))
+@pytest.mark.parametrize("which", sorted(k for k in CONFIGS if k != "M"))   # (M: sizes for the GPU kernels)
 def test_portions_down_to_two_tokens_then_one_by_one(tmp_path, which):
     core, cfg, w = build(tmp_path, which)
     toks = tokens(61, cfg["vocab"], 2)
@@ -53,7 +53,7 @@ def test_portions_down_to_two_tokens_then_one_by_one(tmp_path, which):
     core.storage.manager.check_invariants()
 
 
-@pytest.mark.parametrize("which", sorted(CONFIGS))
+@pytest.mark.parametrize("which", sorted(k for k in CONFIGS if k != "M"))   # (M: sizes for the GPU kernels)
 def test_token_by_token_from_the_first(tmp_path, which):
     core, cfg, w = build(tmp_path, which)
     toks = tokens(20, cfg["vocab"], 3)
@@ -61,7 +61,7 @@ def test_token_by_token_from_the_first(tmp_path, which):
     assert rel_err(got, plain_logits(cfg, w, toks)) < TOL
 
 
-@pytest.mark.parametrize("which", sorted(CONFIGS))
+@pytest.mark.parametrize("which", sorted(k for k in CONFIGS if k != "M"))   # (M: sizes for the GPU kernels)
 def test_unequal_requests_together_with_pages_used_again(tmp_path, which):
     core, cfg, w = build(tmp_path, which, pages=20)     # 160 tokens of room: the third request needs pages given back
     V = cfg["vocab"]

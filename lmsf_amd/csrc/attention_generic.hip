@@ -2,7 +2,8 @@
 // multiple of 4 up to 1024, any page size, float32 or bfloat16 storage, float32 arithmetic.
 //
 // Query token t belongs to request segment seg[t] and stands at position pos[t]. It attends to
-// the keys at positions j in [max(0, pos - window + 1), pos] of that request, read from the pages
+// the keys at positions j in [first_visible_key(pos, window), pos] of that request (a window of the last
+// positions, the query's own chunk of positions, or everything), read from the pages
 // (key j lives in page block_table[seg][j / page_size] at offset j % page_size; K pages are
 // [page, kv_head, offset, d], V pages [page, kv_head, d, offset]). All keys of a step
 // are written to the pages before this kernel runs, so prompts, portions of prompts and single
@@ -39,7 +40,7 @@ __global__ __launch_bounds__(GEN_THREADS) void paged_attention_generic_kernel(
   const int t = blockIdx.x, h = blockIdx.y;
   const int tid = threadIdx.x;
   const int s = seg[t], p = pos[t];
-  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int lo = first_visible_key(p, window);
   const int g = h / (nh / nkv);
   const int* bt = block_tables + (long)s * bt_width;
 
@@ -125,7 +126,6 @@ extern "C" int lmsf_paged_attention_generic(const void* q, long q_stride, void* 
   LMSF_CHECK(num_pages * nkv * ps < 2147483647L, "paged_attention: cache too large for 32-bit row indices");
   LMSF_CHECK(q_stride >= (long)nh * d && out_stride >= (long)nh * d, "paged_attention: row strides too small");
   LMSF_CHECK(nh <= 65535, "paged_attention: too many heads");
-  LMSF_CHECK(window >= 0, "paged_attention: negative window");
   if (n_tokens == 0) return 0;
   const size_t smem = (size_t)(d + 3 * GEN_THREADS) * 4;
   dim3 grid(n_tokens, nh), block(GEN_THREADS);

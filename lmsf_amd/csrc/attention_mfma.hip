@@ -119,7 +119,7 @@ __global__ __launch_bounds__(256) void attn_prefill_mfma_kernel(
     const int tok = t0 + (valid ? t : 0);
     const int p = valid ? pos[tok] : -1;
     rpos[j] = p;
-    rlo[j] = (window > 0 && p >= 0) ? max(0, p - window + 1) : 0;
+    rlo[j] = p >= 0 ? first_visible_key(p, window) : 0;
     const int head = kvh * n_rep + (valid ? hin : 0);
     qoff[j] = (long)tok * q_stride + (long)head * d;
     ooff[j] = (long)tok * out_stride + (long)head * d;
@@ -349,7 +349,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
 
   // the workgroup's range of keys: positions of a tile are consecutive
   const int p_first = pos[t0], p_last = p_first + ntok - 1;
-  const int k_begin = window > 0 ? (max(0, p_first - window + 1) / 32) * 32 : 0;
+  const int k_begin = (first_visible_key(p_first, window) / 32) * 32;
   const int n_steps = (p_last - k_begin) / 32 + 1;
   const int blk0 = k_begin >> ps_log2;                                   // first block of the table that is needed
   const int n_blk = min(btw, (p_last >> ps_log2) + 1) - blk0;             // blocks of the table that are needed
@@ -370,7 +370,7 @@ __global__ __launch_bounds__(NW * 64, (NW == 8 ? 4 : 1)) void attn_prefill_dma_k
     const int tok = t0 + (valid ? t : 0);
     const int p = valid ? p_first + t : -1;
     rpos[j] = p;
-    rlo[j] = (window > 0 && p >= 0) ? max(0, p - window + 1) : 0;
+    rlo[j] = p >= 0 ? first_visible_key(p, window) : 0;
     const int head = kvh * n_rep + (valid ? hin : 0);
     qoff[j] = (long)tok * q_stride + (long)head * d;
     ooff[j] = (long)tok * out_stride + (long)head * d;
@@ -730,7 +730,7 @@ __global__ __launch_bounds__(256) void attn_decode_mfma_kernel(
   const int n_rep = nh / nkv;
   const int tid = threadIdx.x, w = tid >> 6, l = tid & 63, c = l & 15, g = l >> 4;
   const int p = pos[tok];
-  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int lo = first_visible_key(p, window);
   const int c0 = max(split * chunk, (lo / 32) * 32), c1 = min((split + 1) * chunk, p + 1);   // keys [c0, c1)
   if (c0 >= c1) return;
   KvView G;
@@ -927,7 +927,7 @@ __global__ __launch_bounds__(256) void attn_decode_reduce_serial_kernel(
       po[s] = dv < d ? part_o[(base + s) * d + dv] : 0.f;
     }
   }
-  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int lo = first_visible_key(p, window);
   const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);   // splits s0 .. s1 have keys
   float M = -INFINITY;
 #pragma unroll
@@ -954,7 +954,7 @@ __global__ __launch_bounds__(REDUCE_THREADS) void attn_decode_reduce_kernel(
   const int i_tok = blockIdx.x, head = blockIdx.y, tid = threadIdx.x;
   const int tok = tok_idx ? tok_idx[i_tok] : i_tok;
   const int p = pos[tok];
-  const int lo = window > 0 ? max(0, p - window + 1) : 0;
+  const int lo = first_visible_key(p, window);
   const int s0 = ((lo / 32) * 32) / chunk, s1 = min(n_splits - 1, p / chunk);   // splits s0 .. s1 have keys
   const long base = ((long)i_tok * nh + head) * n_splits;
   float M = -INFINITY;
@@ -1010,7 +1010,6 @@ static int check_common(const char* who, const void* q, const void* out, const v
              "%s: row strides must cover nh*d and keep 16-byte (q) and 8-byte (out) alignment", who);
   LMSF_CHECK(lmsf_aligned16(q) && lmsf_aligned16(k_pages) && lmsf_aligned16(v_pages) && lmsf_aligned16(out),
              "%s: operands must be 16-byte aligned", who);
-  LMSF_CHECK(window >= 0, "%s: negative window", who);
   return 0;
 }
 

@@ -146,6 +146,15 @@ __device__ __forceinline__ void rope_rotate(float x, float y, float c, float s, 
   *yr = __fmaf_rn(y, c, __fmul_rn(x, s));
 }
 
+// The first key position that a query at position p attends to; the last is p itself. ``window`` > 0: the last
+// ``window`` positions; < 0: the positions of p's own chunk of -window positions, chunks counted from position 0 of
+// the request (wherever a prompt was cut into steps); 0: every position. It never falls as p rises.
+__device__ __forceinline__ int first_visible_key(int p, int window) {
+  if (window > 0) return max(0, p - window + 1);
+  if (window < 0) return p - p % (-window);
+  return 0;
+}
+
 // ---------------------------------------------------------------- wave64 and block reductions
 
 __device__ __forceinline__ float wave_sum(float v) {

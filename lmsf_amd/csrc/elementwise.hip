@@ -63,6 +63,13 @@ extern "C" int lmsf_patch_tokens(int* ids, const int* src, const int* prev, int 
 // out[t, i] = act(in[t, i]) * in[t, I + i], act computed in float32.
 // kind 0: silu(x) = x / (1 + exp(-x))   (vllm/kernels/activation_kernels.cu:26-42)
 // kind 1: gelu(x) = x/2 (1 + erf(x / sqrt 2)) (vllm/kernels/activation_kernels.cu:44-51)
+// kind 2: the tanh form of gelu, x/2 (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3)))
+template <int KIND>
+__device__ __forceinline__ float gate_activation(float x) {
+  if (KIND == 0) return x / (1.0f + expf(-x));
+  if (KIND == 1) return 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
+  return 0.5f * x * (1.0f + tanhf(0.79788456080286536f * (x + 0.044715f * x * x * x)));
+}
 template <typename T, int KIND>
 __global__ __launch_bounds__(256) void gated_act_kernel(const T* __restrict__ in, T* __restrict__ out, int I,
                                                         long in_stride) {
@@ -71,12 +78,7 @@ __global__ __launch_bounds__(256) void gated_act_kernel(const T* __restrict__ in
   if (i >= I) return;
   const float g = to_f32<T>(in[t * in_stride + i]);
   const float u = to_f32<T>(in[t * in_stride + I + i]);
-  float a;
-  if (KIND == 0)
-    a = g / (1.0f + expf(-g));
-  else
-    a = 0.5f * g * (1.0f + erff(g * 0.70710678118654752f));
-  out[t * (long)I + i] = from_f32<T>(a * u);
+  out[t * (long)I + i] = from_f32<T>(gate_activation<KIND>(g) * u);
 }
 
 // The same with 16-byte accesses: 8 bfloat16 or 4 float32 per thread.
@@ -92,13 +94,7 @@ __global__ __launch_bounds__(256) void gated_act_vec_kernel(const T* __restrict_
   u.load(in + t * in_stride + I + i);
 #pragma unroll
   for (int e = 0; e < N; ++e) {
-    const float x = g.get(e);
-    float a;
-    if (KIND == 0)
-      a = x / (1.0f + expf(-x));
-    else
-      a = 0.5f * x * (1.0f + erff(x * 0.70710678118654752f));
-    o.set(e, a * u.get(e));
+    o.set(e, gate_activation<KIND>(g.get(e)) * u.get(e));
   }
   o.store(out + t * (long)I + i);
 }
@@ -109,7 +105,7 @@ extern "C" int lmsf_gated_act(const void* in, void* out, int dtype, int n_tokens
   LMSF_CHECK(n_tokens >= 0 && I > 0 && in_stride >= 2L * I, "gated_act: bad sizes n=%d I=%d stride=%ld", n_tokens, I,
              in_stride);
   LMSF_CHECK((I + 255) / 256 <= 65535, "gated_act: intermediate size %d too large", I);
-  LMSF_CHECK(kind == 0 || kind == 1, "gated_act: unknown activation %d", kind);
+  LMSF_CHECK(kind >= 0 && kind <= 2, "gated_act: unknown activation %d", kind);
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "gated_act: unknown dtype code %d", dtype);
   if (n_tokens == 0) return 0;
   const int per = dtype == LMSF_F32 ? 4 : 8;   // elements of a 16-byte access
@@ -119,9 +115,9 @@ extern "C" int lmsf_gated_act(const void* in, void* out, int dtype, int n_tokens
 #define GAV(T, K) \
   hipLaunchKernelGGL((gated_act_vec_kernel<T, K>), vgrid, vblock, 0, stream, (const T*)in, (T*)out, I, in_stride)
     if (dtype == LMSF_F32) {
-      if (kind == 0) GAV(float, 0); else GAV(float, 1);
+      if (kind == 0) GAV(float, 0); else if (kind == 1) GAV(float, 1); else GAV(float, 2);
     } else {
-      if (kind == 0) GAV(bf16_t, 0); else GAV(bf16_t, 1);
+      if (kind == 0) GAV(bf16_t, 0); else if (kind == 1) GAV(bf16_t, 1); else GAV(bf16_t, 2);
     }
 #undef GAV
     LMSF_LAUNCH_CHECK("gated_act");
@@ -130,9 +126,9 @@ extern "C" int lmsf_gated_act(const void* in, void* out, int dtype, int n_tokens
   dim3 grid(n_tokens, (I + 255) / 256), block(256);
 #define GA(T, K) hipLaunchKernelGGL((gated_act_kernel<T, K>), grid, block, 0, stream, (const T*)in, (T*)out, I, in_stride)
   if (dtype == LMSF_F32) {
-    if (kind == 0) GA(float, 0); else GA(float, 1);
+    if (kind == 0) GA(float, 0); else if (kind == 1) GA(float, 1); else GA(float, 2);
   } else {
-    if (kind == 0) GA(bf16_t, 0); else GA(bf16_t, 1);
+    if (kind == 0) GA(bf16_t, 0); else if (kind == 1) GA(bf16_t, 1); else GA(bf16_t, 2);
   }
 #undef GA
   LMSF_LAUNCH_CHECK("gated_act");

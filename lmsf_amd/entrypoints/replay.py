@@ -5,11 +5,12 @@ step function, cache manager and kernels that generation uses. The reference has
 it (its closest is the hand-driven step loop of example/examples/llm_engine_example.rs:65-151).
 
     trace_run --model DIR --dtype bfloat16|float32 --out DIR --max-tokens N
-              [--block-size B] [--num-gpu-blocks P] [--random CONFIG.json --seed S]
+              [--block-size B] [--num-gpu-blocks P] [--max-seqs R] [--random CONFIG.json --seed S]
 
 ``--random CONFIG.json`` stands in for ``--model``: the model of that configuration with random weights
 made from ``--seed`` (the engine's random-weights mode). ``--block-size`` is the page size in tokens
-(default 16); ``--num-gpu-blocks`` sets the number of pages instead of deriving it from ``--max-tokens``.
+(default 16); ``--num-gpu-blocks`` sets the number of pages instead of deriving it from ``--max-tokens``;
+``--max-seqs`` is the number of requests that may be live at a time (default 4): the engine has that many state slots.
 
 Steps come on standard input, one JSON object a line:
 
@@ -68,6 +69,8 @@ def main(argv=None) -> int:
     ap.add_argument("--out", required=True, help="folder the logits files are written to")
     ap.add_argument("--max-tokens", type=int, required=True,
                     help="most tokens that live requests hold at any time; the cache pool is made for this many")
+    ap.add_argument("--max-seqs", type=int, default=4,
+                    help="requests that may be live at a time: the engine's state slots (default 4)")
     ap.add_argument("--device", default="cuda:0")
     args = ap.parse_args(argv)
     if args.max_tokens <= 0:
@@ -94,7 +97,7 @@ def main(argv=None) -> int:
     from lmsf_amd.config import load_model_config
     longest = min(load_model_config(model_dir)[1].max_position_embeddings, num_pages * args.block_size)
     core = load_engine_core(model_dir, dtype=args.dtype, block_size=args.block_size, num_pages=num_pages,
-                            max_model_len=longest, max_num_seqs=64, device=args.device, load_format=load_format,
+                            max_model_len=longest, max_num_seqs=max(1, args.max_seqs), device=args.device, load_format=load_format,
                             seed=args.seed)
     _say("model %s ready after %.0f s: %s, %d pages of %d tokens" % (
         core.arch.name, time.time() - t0, args.dtype, num_pages, args.block_size))

@@ -435,8 +435,11 @@ class HipOps:
 
     def paged_attention(self, q: torch.Tensor, k_pages: torch.Tensor, v_pages: torch.Tensor,
                         block_tables: torch.Tensor, seg: torch.Tensor, pos: torch.Tensor, nh: int, nkv: int, d: int,
-                        scale: float, window: int = 0, batch=None, kernel: Optional[str] = None) -> torch.Tensor:
-        """Attention of every query token over the cached keys of its request.
+                        scale: float, window: int = 0, batch=None, kernel: Optional[str] = None,
+                        chunk: int = 0) -> torch.Tensor:
+        """Attention of every query token over the cached keys of its request: those at positions up to its own,
+        within the last ``window`` positions if a window is given, or within its own chunk of ``chunk`` positions
+        (chunks counted from position 0 of the request) if a chunk size is given.
 
         ``q`` is [N, >= nh*d] with unit column stride (it may be the fused QKV buffer, of which the
         first nh*d columns are read). ``k_pages`` [pages, nkv, page_size, d], ``v_pages``
@@ -463,6 +466,10 @@ class HipOps:
         out = torch.empty((N, nh * d), dtype=q.dtype, device=q.device)
         if N == 0:
             return out
+        if chunk:
+            if window or chunk < 0:
+                raise ValueError("paged_attention takes a window or a chunk size (> 0), not both")
+            window = -int(chunk)        # the kernels' encoding of a chunk mask (csrc/common.h: first_visible_key)
         fast_ok = (q.dtype == torch.bfloat16 and d % 16 == 0 and 16 <= d <= 256 and ps % 4 == 0
                    and q.stride(0) % 8 == 0 and q.data_ptr() % 16 == 0 and scale > 0)
         if kernel == "mfma" and not fast_ok:
@@ -744,14 +751,224 @@ class HipOps:
             out.stride(0), N, F, W, _ptr(ints), _ptr(rows), self._stream()))
         return out
 
+    # ------------------------------------------------------------------ Dynamic Tanh, state-carrying mixers
+
+    @staticmethod
+    def _f32_vec(t: torch.Tensor, n: int, name: str) -> None:
+        if t.dtype != torch.float32 or t.numel() != n or not t.is_contiguous():
+            raise ValueError("%s must be contiguous float32 of %d elements" % (name, n))
+
+    def dyt_norm(self, branch: Optional[torch.Tensor], residual: Optional[torch.Tensor], weight: torch.Tensor,
+                 bias: torch.Tensor, alpha: torch.Tensor, out_dtype: torch.dtype,
+                 rows: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """tanh(alpha * r) * weight + bias with r = residual + branch (either may be missing). ``residual``
+        (float32 [N, H]) becomes the sum in place when both are given and ``rows`` is None; ``rows`` (int32 [R])
+        selects rows, the output then has R. ``alpha`` is a float32 tensor of one element."""
+        self._dev(branch, residual, weight, bias, alpha, rows)
+        ref = branch if branch is not None else residual
+        if ref is None or ref.dim() != 2 or not ref.is_contiguous():
+            raise ValueError("dyt_norm needs a contiguous [N, H] branch or residual")
+        N, H = ref.shape
+        if branch is not None and residual is not None and branch.shape != residual.shape:
+            raise ValueError("dyt_norm: branch %s and residual %s differ" % (tuple(branch.shape), tuple(residual.shape)))
+        if residual is not None and (residual.dtype != torch.float32 or not residual.is_contiguous()):
+            raise ValueError("the residual stream must be contiguous float32")
+        self._f32_vec(weight, H, "dyt_norm: weight")
+        self._f32_vec(bias, H, "dyt_norm: bias")
+        self._f32_vec(alpha, 1, "dyt_norm: alpha")
+        self._i32(rows, "rows")
+        n_out = N if rows is None else rows.numel()
+        out = torch.empty((n_out, H), dtype=out_dtype, device=ref.device)
+        self._check(self.lib.lmsf_dyt_norm(_ptr(branch), _code(branch.dtype) if branch is not None else F32,
+                                           _ptr(residual), _ptr(weight), _ptr(bias), _ptr(alpha), _ptr(out),
+                                           _code(out_dtype), _ptr(rows), n_out, H, self._stream()))
+        return out
+
+    def _segments(self, batch, n_tokens: int):
+        """(seg_of, seg_starts, state_slots, segments) of a step, checked."""
+        self._dev(batch.seg_of_token, batch.seg_starts, batch.state_slots)
+        S = batch.n_segments
+        self._i32(batch.seg_of_token, "seg_of_token", n_tokens)
+        self._i32(batch.seg_starts, "seg_starts", S + 1)
+        self._i32(batch.state_slots, "state_slots", S)
+        return batch.seg_of_token, batch.seg_starts, batch.state_slots, S
+
+    @staticmethod
+    def _state_view(state: torch.Tensor, need: int, name: str) -> None:
+        if state.dtype != torch.float32 or state.dim() != 2 or state.stride(1) != 1 or state.shape[1] < need \
+                or not state.is_cuda:
+            raise ValueError("%s: the state must be float32 [slots, >= %d] with unit column stride" % (name, need))
+
+    def short_conv(self, u: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor], state: Optional[torch.Tensor],
+                   batch, activation: Optional[str] = None) -> torch.Tensor:
+        """Causal convolution over time, channel by channel: out[t, c] = act(bias[c] + sum_j weight[c, j] u[t - taps + 1 + j, c])
+        within each request. ``u`` [N, C] (a view with unit column stride will do), ``weight`` [C, taps]; ``state``
+        float32 [slots, >= C (taps - 1)] holds every request's last taps - 1 inputs and is brought up to date.
+        ``batch`` is the step (engine.batch.StepContext). activation None or "silu"."""
+        self._dev(u, weight, bias)
+        if u.dim() != 2 or u.stride(1) != 1 or weight.dim() != 2 or weight.shape[0] != u.shape[1] \
+                or not weight.is_contiguous() or weight.dtype != u.dtype:
+            raise ValueError("short_conv: u [N, C] and weight [C, taps] of one dtype are needed")
+        N, C = u.shape
+        taps = weight.shape[1]
+        if bias is not None and (bias.shape != (C,) or bias.dtype != u.dtype or not bias.is_contiguous()):
+            raise ValueError("short_conv: bias must be [%d] of u's dtype" % C)
+        if activation not in (None, "silu"):
+            raise ValueError("short_conv: activation %r unknown (None, silu)" % (activation,))
+        if taps > 1:
+            if state is None:
+                raise ValueError("short_conv: a convolution over %d taps needs a state" % taps)
+            self._state_view(state, C * (taps - 1), "short_conv")
+        seg_of, seg_starts, slots, S = self._segments(batch, N)
+        out = torch.empty((N, C), dtype=u.dtype, device=u.device)
+        self._check(self.lib.lmsf_short_conv(
+            _ptr(u), _code(u.dtype), u.stride(0), _ptr(weight), _ptr(bias), 1 if activation else 0, _ptr(state),
+            state.stride(0) if state is not None else 0, _ptr(seg_of), _ptr(seg_starts), _ptr(slots), _ptr(out),
+            out.stride(0), N, S, C, taps, self._stream()))
+        return out
+
+    def selective_scan(self, x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, b_at: int, c_at: int, z: torch.Tensor,
+                       a_log: torch.Tensor, d_skip: torch.Tensor, state: torch.Tensor, batch) -> torch.Tensor:
+        """The selective scan over each request's tokens, the state carried in ``state`` (float32
+        [slots, >= inner * n]): S[c, n] <- exp(dt_c A[c, n]) S[c, n] + dt_c x_c B_n, y_c = (sum_n S[c, n] C_n + D_c x_c)
+        silu(z_c), with dt = softplus(``dt``) (float32 [N, inner], before the softplus), A = -exp(``a_log``)
+        (float32 [inner, n]), B = bc[:, b_at:b_at + n], C = bc[:, c_at:c_at + n]. x, z, bc: views with unit column
+        stride, one dtype. Returns y [N, inner] in x's dtype."""
+        self._dev(x, dt, bc, z, a_log, d_skip)
+        N, inner = x.shape
+        if a_log.dim() != 2 or a_log.shape[0] != inner or a_log.dtype != torch.float32 or not a_log.is_contiguous():
+            raise ValueError("selective_scan: a_log must be contiguous float32 [%d, n]" % inner)
+        n = a_log.shape[1]
+        self._f32_vec(d_skip, inner, "selective_scan: D")
+        if dt.dtype != torch.float32 or tuple(dt.shape) != (N, inner) or dt.stride(1) != 1:
+            raise ValueError("selective_scan: dt must be float32 [%d, %d]" % (N, inner))
+        for t, w, name in ((x, inner, "x"), (z, inner, "z"), (bc, max(b_at, c_at) + n, "bc")):
+            if t.dim() != 2 or t.shape[0] != N or t.shape[1] < w or t.stride(1) != 1 or t.dtype != x.dtype:
+                raise ValueError("selective_scan: %s must be [%d, >= %d] of x's dtype with unit column stride" % (name, N, w))
+        self._state_view(state, inner * n, "selective_scan")
+        _, seg_starts, slots, S = self._segments(batch, N)
+        y = torch.empty((N, inner), dtype=x.dtype, device=x.device)
+        self._check(self.lib.lmsf_selective_scan(
+            _ptr(x), _code(x.dtype), x.stride(0), _ptr(dt), dt.stride(0), _ptr(bc), bc.stride(0), int(b_at), int(c_at),
+            _ptr(z), z.stride(0), _ptr(a_log), _ptr(d_skip), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots),
+            _ptr(y), y.stride(0), N, S, inner, n, self._stream()))
+        return y
+
+    def mlstm_state_floats(self, heads: int, dim: int, vdim: int) -> int:
+        return int(self.lib.lmsf_mlstm_state_floats(heads, dim, vdim))
+
+    def mlstm(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, gates: torch.Tensor, out_gate: torch.Tensor,
+              norm_weight: torch.Tensor, state: torch.Tensor, batch, heads: int, dim: int, vdim: int, q_scale: float,
+              gate_cap: float, eps: float) -> torch.Tensor:
+        """A matrix memory per head with exponential gates, over each request's tokens, the memory carried in
+        ``state`` (csrc/recurrent.hip says how it is laid out and what is computed). q, k [N, heads * dim] and v
+        [N, heads * vdim]: views of one buffer (equal row strides); ``gates`` float32 [N, 2 heads]: the input gates'
+        pre-activations, then the forget gates'; ``out_gate`` [N, heads * vdim] before its sigmoid; ``norm_weight``
+        float32 [heads * vdim]. Returns [N, heads * vdim] in q's dtype: every head's output over its root mean
+        square, times the weight, times the gate."""
+        self._dev(q, k, v, gates, out_gate, norm_weight)
+        N = q.shape[0]
+        for t, w, name in ((q, heads * dim, "q"), (k, heads * dim, "k"), (v, heads * vdim, "v"),
+                           (out_gate, heads * vdim, "out_gate")):
+            if t.dim() != 2 or t.shape[0] != N or t.shape[1] < w or t.stride(1) != 1 or t.dtype != q.dtype:
+                raise ValueError("mlstm: %s must be [%d, >= %d] of q's dtype with unit column stride" % (name, N, w))
+        if not (q.stride(0) == k.stride(0) == v.stride(0)):
+            raise ValueError("mlstm: q, k and v must have one row stride")
+        if gates.dtype != torch.float32 or tuple(gates.shape) != (N, 2 * heads) or gates.stride(1) != 1:
+            raise ValueError("mlstm: gates must be float32 [%d, %d]" % (N, 2 * heads))
+        self._f32_vec(norm_weight, heads * vdim, "mlstm: norm weight")
+        self._state_view(state, self.mlstm_state_floats(heads, dim, vdim), "mlstm")
+        _, seg_starts, slots, S = self._segments(batch, N)
+        out = torch.empty((N, heads * vdim), dtype=q.dtype, device=q.device)
+        self._check(self.lib.lmsf_mlstm(
+            _ptr(q), _ptr(k), _ptr(v), _code(q.dtype), q.stride(0), _ptr(gates), gates.stride(0), _ptr(out_gate),
+            out_gate.stride(0), _ptr(norm_weight), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots), _ptr(out),
+            out.stride(0), N, S, int(heads), int(dim), int(vdim), float(q_scale), float(gate_cap), float(eps),
+            self._stream()))
+        return out
+
+    # ------------------------------------------------------------------ attention with keys and values of two sizes
+
+    def attn_prepare(self, q: torch.Tensor, k: torch.Tensor, v: torch.Tensor, heads: int, kv_heads: int, dim: int,
+                     vdim: int, padded: int, positions: torch.Tensor, slots: Optional[torch.Tensor],
+                     k_pages: Optional[torch.Tensor], v_pages: Optional[torch.Tensor], table: Optional[torch.Tensor] = None,
+                     unit_norm_eps: Optional[float] = None, temp_coef: float = 0.0, temp_every: int = 0) -> torch.Tensor:
+        """Readies projected queries, keys and values for ``paged_attention`` at head size ``padded``: q and k are
+        (each step optional) divided by their root mean square over the head (``unit_norm_eps``), rotated by the
+        position over the first table.shape[1] entries in pairs (i, i + rot/2) (``table`` float32 [max_pos, rot] =
+        [cos | sin]), q is multiplied by 1 + temp_coef ln(floor((p + 1) / temp_every) + 1); k and v go to the
+        tokens' slots of the pages, everything padded with zeros to ``padded`` entries a head. q [N, heads * dim],
+        k [N, kv_heads * dim], v [N, kv_heads * vdim]: views with unit column stride. Returns q [N, heads * padded]."""
+        self._dev(q, k, v, positions, slots, k_pages, v_pages, table)
+        N = q.shape[0]
+        for t, w, name in ((q, heads * dim, "q"), (k, kv_heads * dim, "k"), (v, kv_heads * vdim, "v")):
+            if t.dim() != 2 or t.shape[0] != N or t.shape[1] < w or t.stride(1) != 1 or t.dtype != q.dtype:
+                raise ValueError("attn_prepare: %s must be [%d, >= %d] of q's dtype with unit column stride" % (name, N, w))
+        self._i32(positions, "positions", N)
+        rot = max_pos = 0
+        if table is not None:
+            if table.dtype != torch.float32 or table.dim() != 2 or not table.is_contiguous() or table.shape[1] > dim \
+                    or table.shape[1] % 2:
+                raise ValueError("attn_prepare: the rotary table must be contiguous float32 [max_pos, rot <= %d]" % dim)
+            max_pos, rot = table.shape
+        num_pages, ps = 0, 1
+        if slots is not None:
+            self._i32(slots, "slots", N)
+            if k_pages is None or k_pages.dim() != 4 or k_pages.shape[1] != kv_heads or k_pages.shape[3] != padded \
+                    or not k_pages.is_contiguous() or k_pages.dtype != q.dtype:
+                raise ValueError("attn_prepare: k_pages must be contiguous [pages, %d, page_size, %d] of %s"
+                                 % (kv_heads, padded, q.dtype))
+            num_pages, ps = k_pages.shape[0], k_pages.shape[2]
+            if v_pages is None or tuple(v_pages.shape) != (num_pages, kv_heads, padded, ps) or not v_pages.is_contiguous() \
+                    or v_pages.dtype != q.dtype:
+                raise ValueError("attn_prepare: v_pages must be contiguous [%d, %d, %d, %d] of %s"
+                                 % (num_pages, kv_heads, padded, ps, q.dtype))
+        out = torch.empty((N, heads * padded), dtype=q.dtype, device=q.device)
+        self._check(self.lib.lmsf_attn_prepare(
+            _ptr(q), q.stride(0), _ptr(k), k.stride(0), _ptr(v), v.stride(0), _code(q.dtype), _ptr(positions), _ptr(table),
+            rot, max_pos, _ptr(slots), _ptr(out), out.stride(0), _ptr(k_pages), _ptr(v_pages), num_pages, N, int(heads),
+            int(kv_heads), int(dim), int(vdim), int(padded), ps, 0 if unit_norm_eps is None else 1,
+            float(unit_norm_eps or 0.0), float(temp_coef), int(temp_every), self._stream()))
+        return out
+
+    def head_gate(self, x: torch.Tensor, x_head: int, heads: int, vdim: int, gate: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """out[n, h * vdim + e] = x[n, h * x_head + e] * sigmoid(gate[n, h * vdim + e]) (no gate: the copy that drops
+        what lies behind every head's first ``vdim`` entries)."""
+        self._dev(x, gate)
+        N = x.shape[0]
+        if x.dim() != 2 or x.stride(1) != 1 or x.shape[1] < (heads - 1) * x_head + vdim or x_head < vdim:
+            raise ValueError("head_gate: x too narrow for %d heads of %d" % (heads, x_head))
+        if gate is not None and (gate.dim() != 2 or gate.shape[0] != N or gate.shape[1] < heads * vdim or gate.stride(1) != 1
+                                 or gate.dtype != x.dtype):
+            raise ValueError("head_gate: gate must be [%d, >= %d] of x's dtype" % (N, heads * vdim))
+        out = torch.empty((N, heads * vdim), dtype=x.dtype, device=x.device)
+        self._check(self.lib.lmsf_head_gate(_ptr(x), _code(x.dtype), x.stride(0), int(x_head), _ptr(gate),
+                                            gate.stride(0) if gate is not None else 0, _ptr(out), out.stride(0), N,
+                                            int(heads), int(vdim), self._stream()))
+        return out
+
+    def rms_pair(self, a: torch.Tensor, b: torch.Tensor, wa: torch.Tensor, wb: torch.Tensor, eps: float,
+                 scale: float = 0.5) -> torch.Tensor:
+        """scale * (a / rms(a) * wa + b / rms(b) * wb), row by row; a, b [N, W] of one dtype, the weights float32."""
+        self._dev(a, b, wa, wb)
+        if a.dim() != 2 or a.shape != b.shape or a.dtype != b.dtype or a.stride(1) != 1 or b.stride(1) != 1:
+            raise ValueError("rms_pair: a and b must be [N, W] of one dtype with unit column stride")
+        N, W = a.shape
+        self._f32_vec(wa, W, "rms_pair: first weight")
+        self._f32_vec(wb, W, "rms_pair: second weight")
+        out = torch.empty((N, W), dtype=a.dtype, device=a.device)
+        self._check(self.lib.lmsf_rms_pair(_ptr(a), a.stride(0), _ptr(b), b.stride(0), _code(a.dtype), _ptr(wa), _ptr(wb),
+                                           _ptr(out), N, W, float(eps), float(scale), self._stream()))
+        return out
+
     # ------------------------------------------------------------------ feed-forward
 
     def gated_act(self, gu: torch.Tensor, kind: str = "silu") -> torch.Tensor:
-        """act(gu[:, :I]) * gu[:, I:] for gu [N, 2I]; kind "silu" or "gelu"."""
+        """act(gu[:, :I]) * gu[:, I:] for gu [N, 2I]; kind "silu", "gelu" (erf form) or "gelu_tanh"."""
         self._dev(gu)
         if gu.dim() != 2 or gu.stride(1) != 1 or gu.shape[1] % 2 != 0:
             raise ValueError("gated_act input must be [N, 2I] with unit column stride")
-        kinds = {"silu": 0, "gelu": 1}
+        kinds = {"silu": 0, "gelu": 1, "gelu_tanh": 2}
         if kind not in kinds:
             raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))
         N, I = gu.shape[0], gu.shape[1] // 2
@@ -844,6 +1061,9 @@ class HipOps:
         split K over 8 and over 16 waves). ``x`` may be a ``ScaledRows``."""
         if weight.dim() != 2 or weight.shape[0] % 2 != 0:
             raise ValueError("linear_gated: weight must be [2 I, K]")
+        if kind == "gelu_tanh":
+            # (no product has this activation as its epilogue: the product, then the activation kernel)
+            return self.gated_act(self.linear(self.materialize(x), weight, bias), kind)
         kinds = {"silu": 1, "gelu": 2}
         if kind not in kinds:
             raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))

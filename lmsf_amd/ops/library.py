@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 26
+ABI_VERSION = 27
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -51,6 +51,19 @@ _SIGNATURES = {
                                c_long, c_int, c_int, c_int, _P, _P, _P]),
     "lmsf_table_moe_scratch_ints": (c_long, [c_int, c_int, c_int]),
     "lmsf_table_moe_grouped": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_long]),
+    "lmsf_dyt_norm": (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P]),
+    "lmsf_short_conv": (c_int, [_P, c_int, c_long, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, c_long, c_int, c_int, c_int,
+                                c_int, _P]),
+    "lmsf_selective_scan": (c_int, [_P, c_int, c_long, _P, c_long, _P, c_long, c_int, c_int, _P, c_long, _P, _P, _P,
+                                    c_long, _P, _P, _P, c_long, c_int, c_int, c_int, c_int, _P]),
+    "lmsf_mlstm_state_floats": (c_long, [c_int, c_int, c_int]),
+    "lmsf_mlstm": (c_int, [_P, _P, _P, c_int, c_long, _P, c_long, _P, c_long, _P, _P, c_long, _P, _P, _P, c_long, c_int,
+                           c_int, c_int, c_int, c_int, c_float, c_float, c_float, _P]),
+    "lmsf_attn_prepare": (c_int, [_P, c_long, _P, c_long, _P, c_long, c_int, _P, _P, c_int, c_int, _P, _P, c_long, _P, _P,
+                                  c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
+                                  _P]),
+    "lmsf_head_gate": (c_int, [_P, c_int, c_long, c_int, _P, c_long, _P, c_long, c_int, c_int, c_int, _P]),
+    "lmsf_rms_pair": (c_int, [_P, c_long, _P, c_long, c_int, _P, _P, _P, c_int, c_int, c_float, c_float, _P]),
     "lmsf_gated_act": (c_int, [_P, _P, c_int, c_int, c_int, c_long, c_int, _P]),
     "lmsf_gemm_plain": (c_int, [_P, c_int, c_long, _P, c_int, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, _P]),
     "lmsf_gemm_skinny": (c_int, [_P, c_long, _P, c_long, _P, _P, c_int, c_long, c_int, c_int, c_int, c_int, c_int, _P]),

@@ -87,7 +87,8 @@ class TensorDecl:
     compute in float32 anyway and take the weight as it is); the matrices of the products are cast as the
     reference casts everything (core/src/model_executor/models/model_factory.rs:124-139). ``init`` says how
     the random-weights mode fills it: "normal" (mean 0, the mode's standard deviation), "ones", "zeros", "last_one"
-    (zeros and a final 1) or, for an integer table, "choices:E" (every row distinct numbers below E)."""
+    (zeros and a final 1), "const:x" (every entry x), "normal:s" (standard deviation s whatever the mode's) or, for an
+    integer table, "choices:E" (every row distinct numbers below E)."""
 
     shape: Tuple[int, ...]
     kind: str = "float"

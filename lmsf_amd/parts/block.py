@@ -16,11 +16,19 @@ class PreNormResidualBlock(Block):
     Where the norm that follows accepts it, the o and down products may stay unfinished
     (``PendingProduct``) and the norm's kernel adds up their partial sums; where a norm may defer
     its work and the part after it takes that, the norm runs inside that part's first product.
+    A layer without a feed-forward (a part that says ``absent``) has only the first sublayer and needs no
+    "post_mixer" norm: the mixer's output is what the block returns, not yet added.
     """
 
     graph_safe = True
 
-    ROLES = ("input", "post_mixer")
+    ROLES = ("input",)          # and "post_mixer" where there is a feed-forward
+
+    def __init__(self, prefix: str, rt, mixer, feed_forward, norms):
+        super().__init__(prefix, rt, mixer, feed_forward, norms)
+        self.has_ffn = not getattr(feed_forward, "absent", False)
+        if self.has_ffn and "post_mixer" not in norms:
+            raise ValueError("block %s needs the norm post_mixer before its feed-forward" % prefix)
 
     @property
     def accepts_pending_branch(self) -> bool:
@@ -28,11 +36,15 @@ class PreNormResidualBlock(Block):
 
     def forward(self, branch: Optional[torch.Tensor], residual: torch.Tensor, ctx,
                 binding: CacheBinding) -> torch.Tensor:
-        first, post = self.norms["input"], self.norms["post_mixer"]
+        first, post = self.norms["input"], self.norms.get("post_mixer")
         if first.may_defer and self.mixer.accepts_normed:
             h = first.forward_add(branch, residual, defer_ok=True)
         else:
             h = first.forward_add(branch, residual)
+        if not self.has_ffn:
+            if self.mixer.may_return_pending and self.pending_output_ok:
+                return self.mixer.forward(h, ctx, binding, pending_ok=True)
+            return self.mixer.forward(h, ctx, binding)
         if self.mixer.may_return_pending and post.accepts_pending:
             a = self.mixer.forward(h, ctx, binding, pending_ok=True)
         else:

@@ -17,34 +17,43 @@ class FusedLinear(Part):
 
     ``sources`` is a list of (checkpoint sub-name, rows): the tensor ``prefix.sub-name.weight`` has
     shape [rows, in_features] and, with ``bias``, ``prefix.sub-name.bias`` has [rows]. With ``bare_names`` the
-    matrix is the tensor ``prefix.sub-name`` itself (checkpoints that name a matrix without ".weight")."""
+    matrix is the tensor ``prefix.sub-name`` itself (checkpoints that name a matrix without ".weight").
+    ``bias`` may also list the sub-names that have a bias (the others' rows of the fused bias are zeros);
+    ``bias_name`` is what a bias is called after its matrix's name ("bias", or "b")."""
 
     graph_safe = True
 
     def __init__(self, prefix: str, rt: Runtime, in_features: int, sources: Sequence[Tuple[str, int]],
-                 bias: bool = False, bare_names: bool = False):
+                 bias=False, bare_names: bool = False, bias_name: str = "bias"):
         super().__init__(prefix, rt)
         self.bare_names = bool(bare_names)
+        self.bias_name = str(bias_name)
+        self.biased = None if isinstance(bias, bool) else set(str(b) for b in bias)   # None: all or none
         if not sources:
             raise ValueError("FusedLinear needs at least one source")
         self.in_features = int(in_features)
         self.sources = [(str(n), int(r)) for n, r in sources]
         self.out_features = sum(r for _, r in self.sources)
-        self.has_bias = bool(bias)
+        self.has_bias = bool(bias) if isinstance(bias, bool) else bool(self.biased)
         self.weight: Optional[torch.Tensor] = None
         self.bias: Optional[torch.Tensor] = None
 
     def _name(self, sub: str, what: str) -> str:
         if self.bare_names and what == "weight":
             return "%s.%s" % (self.prefix, sub) if self.prefix else sub
+        if what == "bias":
+            what = self.bias_name
         return "%s.%s.%s" % (self.prefix, sub, what) if self.prefix else "%s.%s" % (sub, what)
+
+    def _has_bias(self, sub: str) -> bool:
+        return self.has_bias and (self.biased is None or sub in self.biased)
 
     def checkpoint_tensors(self) -> Dict[str, TensorDecl]:
         out = {}
         for sub, rows in self.sources:
             out[self._name(sub, "weight")] = TensorDecl((rows, self.in_features))
-            if self.has_bias:
-                out[self._name(sub, "bias")] = TensorDecl((rows,))
+            if self._has_bias(sub):
+                out[self._name(sub, "bias")] = TensorDecl((rows,), init="zeros")
         return out
 
     def _buffer(self, what: str, dtype: torch.dtype, device) -> torch.Tensor:
@@ -68,6 +77,10 @@ class FusedLinear(Part):
         out = self._buffer(what, self.rt.dtype, self.rt.device)
         row = 0
         for sub, rows in self.sources:
+            if what == "bias" and not self._has_bias(sub):
+                out[row:row + rows].zero_()
+                row += rows
+                continue
             t = fetch(self._name(sub, what))
             if (t.dtype != out.dtype and t.dtype == torch.float32) or t.device != out.device:
                 # a source stored in 32 bits: the buffer takes the widest type (and lies where the sources lie)
@@ -94,5 +107,5 @@ class Linear(FusedLinear):
     """A single checkpoint matrix ``prefix.name.weight`` [out_features, in_features]."""
 
     def __init__(self, prefix: str, rt: Runtime, name: str, in_features: int, out_features: int, bias: bool = False,
-                 bare_names: bool = False):
-        super().__init__(prefix, rt, in_features, [(name, out_features)], bias, bare_names)
+                 bare_names: bool = False, bias_name: str = "bias"):
+        super().__init__(prefix, rt, in_features, [(name, out_features)], bias, bare_names, bias_name)

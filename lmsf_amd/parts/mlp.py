@@ -1,4 +1,4 @@
-"""Gated feed-forward: y = (act(x Wg^T) * (x Wu^T)) Wd^T.
+"""Gated feed-forward: y = (act(x Wg^T) * (x Wu^T)) Wd^T; act is SiLU, GELU or the tanh form of GELU.
 
 core/src/model_executor/models/llama/llama.rs:223-274: gate and up are one fused product of 2 I
 rows (gate first), then silu_and_mul (vllm/kernels/activation_kernels.cu:26-42), then down.
@@ -17,8 +17,8 @@ class GatedMLP(FeedForward):
                  bias: bool = False, gate_name: str = "gate_proj", up_name: str = "up_proj",
                  down_name: str = "down_proj", bare_names: bool = False):
         super().__init__(prefix, rt)
-        if activation not in ("silu", "gelu"):
-            raise ValueError("gated_mlp activation %r unknown (silu, gelu)" % activation)
+        if activation not in ("silu", "gelu", "gelu_tanh"):
+            raise ValueError("gated_mlp activation %r unknown (silu, gelu, gelu_tanh)" % activation)
         self.activation = activation
         self.gate_up = FusedLinear(prefix, rt, hidden_size,
                                    [(gate_name, intermediate_size), (up_name, intermediate_size)], bias=bias,

@@ -50,7 +50,11 @@ def random_tensor(name: str, decl: TensorDecl, seed: int, std: float, dtype: tor
         t = torch.zeros(decl.shape, dtype=dtype, device=device)
         t.reshape(-1)[-1] = 1
         return t
-    if decl.init != "normal":
+    if decl.init.startswith("const:"):
+        return torch.full(decl.shape, float(decl.init.split(":")[1]), dtype=dtype, device=device)
+    if decl.init.startswith("normal:"):
+        std = float(decl.init.split(":")[1])        # a standard deviation of the tensor's own
+    elif decl.init != "normal":
         raise ValueError("tensor %r: unknown init %r" % (name, decl.init))
     gen = torch.Generator(device=device)
     gen.manual_seed(tensor_seed(seed, name))

@@ -124,7 +124,8 @@ class TorchOps:
         return y
 
     # ------------------------------------------------------------ attention
-    def paged_attention(self, q, k_pages, v_pages, block_tables, seg, pos, nh, nkv, d, scale, window=0, batch=None):
+    def paged_attention(self, q, k_pages, v_pages, block_tables, seg, pos, nh, nkv, d, scale, window=0, batch=None,
+                        kernel=None, chunk=0):
         N = q.shape[0]
         ps = k_pages.shape[2]
         out = torch.empty((N, nh * d), dtype=q.dtype, device=q.device)
@@ -132,6 +133,8 @@ class TorchOps:
         for t in range(N):
             s, p = int(seg[t]), int(pos[t])
             lo = max(0, p - window + 1) if window and window > 0 else 0
+            if chunk:
+                lo = p - p % chunk
             js = torch.arange(lo, p + 1, device=q.device)
             pages = block_tables[s].long()[js // ps]
             keys = k_pages[pages, :, js % ps, :].to(torch.float32)      # [n, nkv, d]
@@ -229,6 +232,130 @@ class TorchOps:
             out = out + base.to(torch.float32)
         return out.to(h.dtype)
 
+    # ------------------------------------------------------------ Dynamic Tanh, state-carrying mixers
+    def dyt_norm(self, branch, residual, weight, bias, alpha, out_dtype, rows=None):
+        x = None
+        if branch is not None:
+            x = branch.to(torch.float32)
+        if residual is not None:
+            x = residual if x is None else x + residual
+        if branch is not None and residual is not None and rows is None:
+            residual.copy_(x)
+        if rows is not None:
+            x = x[rows.long()]
+        return (torch.tanh(alpha * x) * weight + bias).to(out_dtype)
+
+    @staticmethod
+    def _segments(batch):
+        starts = [int(v) for v in batch.seg_starts[:batch.n_segments + 1]]
+        slots = [int(v) for v in batch.state_slots[:batch.n_segments]]
+        return [(starts[i], starts[i + 1], slots[i]) for i in range(batch.n_segments)]
+
+    def short_conv(self, u, weight, bias, state, batch, activation=None):
+        C, taps = weight.shape
+        w = weight.to(torch.float32)
+        out = torch.empty((u.shape[0], C), dtype=u.dtype)
+        for a, b, slot in self._segments(batch):
+            old = state[slot, :C * (taps - 1)].reshape(C, taps - 1).t() if taps > 1 else torch.zeros(0, C)
+            seq = torch.cat([old, u[a:b].to(torch.float32)], 0)             # [taps - 1 + n, C]
+            y = sum(seq[j:j + (b - a)] * w[:, j] for j in range(taps))
+            if bias is not None:
+                y = y + bias.to(torch.float32)
+            if activation == "silu":
+                y = y / (1.0 + torch.exp(-y))
+            out[a:b] = y.to(u.dtype)
+            if taps > 1:
+                state[slot, :C * (taps - 1)] = seq[seq.shape[0] - (taps - 1):].t().reshape(-1)
+        return out
+
+    def selective_scan(self, x, dt, bc, b_at, c_at, z, a_log, d_skip, state, batch):
+        inner, n = a_log.shape
+        A = -torch.exp(a_log)
+        y = torch.empty((x.shape[0], inner), dtype=x.dtype)
+        for a, b, slot in self._segments(batch):
+            S = state[slot, :inner * n].reshape(inner, n).clone()
+            for t in range(a, b):
+                d = torch.nn.functional.softplus(dt[t], threshold=20.0)
+                xt, zt = x[t].to(torch.float32), z[t, :inner].to(torch.float32)
+                B, Cc = bc[t, b_at:b_at + n].to(torch.float32), bc[t, c_at:c_at + n].to(torch.float32)
+                S = torch.exp(d[:, None] * A) * S + (d * xt)[:, None] * B[None, :]
+                y[t] = ((S @ Cc + d_skip * xt) * (zt / (1.0 + torch.exp(-zt)))).to(x.dtype)
+            state[slot, :inner * n] = S.reshape(-1)
+        return y
+
+    def mlstm_state_floats(self, heads, dim, vdim):
+        return heads * dim * (vdim + 1) + heads
+
+    def mlstm(self, q, k, v, gates, out_gate, norm_weight, state, batch, heads, dim, vdim, q_scale, gate_cap, eps):
+        H, d, dv = heads, dim, vdim
+        out = torch.empty((q.shape[0], H * dv), dtype=q.dtype)
+        nS = H * d * (dv + 1)
+        for a, b, slot in self._segments(batch):
+            Sx = state[slot, :nS].reshape(H, d, dv + 1).clone()              # S, and n as the last column
+            m = state[slot, nS:nS + H].clone()
+            for t in range(a, b):
+                qt = q[t, :H * d].to(torch.float32).reshape(H, d) * q_scale
+                kt = k[t, :H * d].to(torch.float32).reshape(H, d)
+                vt = torch.cat([v[t, :H * dv].to(torch.float32).reshape(H, dv), torch.ones(H, 1)], 1)
+                gi = gate_cap * torch.tanh(gates[t, :H] / gate_cap)
+                gf = torch.nn.functional.logsigmoid(gate_cap * torch.tanh(gates[t, H:2 * H] / gate_cap))
+                m_new = torch.maximum(gf + m, gi)
+                keep, take = torch.exp(gf + m - m_new), torch.exp(gi - m_new)
+                m = m_new
+                Sx = keep[:, None, None] * Sx + take[:, None, None] * kt[:, :, None] * vt[:, None, :]
+                ox = torch.einsum("hdv,hd->hv", Sx, qt)
+                o = ox[:, :dv] / (torch.maximum(ox[:, dv].abs(), torch.exp(-m)) + 1e-6)[:, None]
+                o = o / torch.sqrt((o * o).mean(-1, keepdim=True) + eps)
+                g = out_gate[t, :H * dv].to(torch.float32)
+                out[t] = (o.reshape(-1) * norm_weight * torch.sigmoid(g)).to(q.dtype)
+            state[slot, :nS] = Sx.reshape(-1)
+            state[slot, nS:nS + H] = m
+        return out
+
+    def attn_prepare(self, q, k, v, heads, kv_heads, dim, vdim, padded, positions, slots, k_pages, v_pages, table=None,
+                     unit_norm_eps=None, temp_coef=0.0, temp_every=0):
+        N = q.shape[0]
+        qf = q[:, :heads * dim].to(torch.float32).reshape(N, heads, dim)
+        kf = k[:, :kv_heads * dim].to(torch.float32).reshape(N, kv_heads, dim)
+        if unit_norm_eps is not None:
+            qf = qf / torch.sqrt((qf * qf).mean(-1, keepdim=True) + unit_norm_eps)
+            kf = kf / torch.sqrt((kf * kf).mean(-1, keepdim=True) + unit_norm_eps)
+        if table is not None:
+            rot = table.shape[1]
+            cs = table[positions.long()][:, None, :]
+            qf = torch.cat([self._rotate(qf[..., :rot], cs, rot), qf[..., rot:]], -1)
+            kf = torch.cat([self._rotate(kf[..., :rot], cs, rot), kf[..., rot:]], -1)
+        if temp_every:
+            p = positions.to(torch.float32)
+            qf = qf * (1.0 + temp_coef * torch.log(torch.floor((p + 1) / temp_every) + 1.0))[:, None, None]
+        out = torch.zeros((N, heads, padded), dtype=q.dtype)
+        out[..., :dim] = qf.to(q.dtype)
+        if slots is not None:
+            ps = k_pages.shape[2]
+            sl = slots.long()
+            ok = sl >= 0
+            page, off = sl[ok] // ps, sl[ok] % ps
+            kp = torch.zeros((N, kv_heads, padded), dtype=q.dtype)
+            kp[..., :dim] = kf.to(q.dtype)
+            vp = torch.zeros((N, kv_heads, padded), dtype=q.dtype)
+            vp[..., :vdim] = v[:, :kv_heads * vdim].reshape(N, kv_heads, vdim)
+            k_pages[page, :, off, :] = kp[ok]
+            v_pages[page, :, :, off] = vp[ok]
+        return out.reshape(N, heads * padded)
+
+    def head_gate(self, x, x_head, heads, vdim, gate=None):
+        N = x.shape[0]
+        y = x[:, :heads * x_head].reshape(N, heads, x_head)[..., :vdim].reshape(N, heads * vdim).to(torch.float32)
+        if gate is not None:
+            y = y * torch.sigmoid(gate[:, :heads * vdim].to(torch.float32))
+        return y.to(x.dtype)
+
+    def rms_pair(self, a, b, wa, wb, eps, scale=0.5):
+        a32, b32 = a.to(torch.float32), b.to(torch.float32)
+        na = a32 / torch.sqrt((a32 * a32).mean(-1, keepdim=True) + eps) * wa
+        nb = b32 / torch.sqrt((b32 * b32).mean(-1, keepdim=True) + eps) * wb
+        return (scale * (na + nb)).to(a.dtype)
+
     # ------------------------------------------------------------ feed-forward / linear
     def gated_act(self, gu, kind="silu"):
         I = gu.shape[1] // 2
@@ -237,6 +364,8 @@ class TorchOps:
             a = g / (1.0 + torch.exp(-g))
         elif kind == "gelu":
             a = 0.5 * g * (1.0 + torch.erf(g / math.sqrt(2.0)))
+        elif kind == "gelu_tanh":
+            a = 0.5 * g * (1.0 + torch.tanh(math.sqrt(2.0 / math.pi) * (g + 0.044715 * g * g * g)))
         else:
             raise ValueError(kind)
         return (a * u).to(gu.dtype)

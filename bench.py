@@ -434,15 +434,51 @@ def takosun_shapes(name):
     return tako, llama
 
 
+def niresun_shapes(name):
+    """A Niresun configuration at sizes that resemble a real model's layers, and the Llama configuration of equal
+    width, depth, heads and feed-forward size beside it. The layers go round selective scan (no feed-forward),
+    chunked gated attention, selective scan, attention beside a matrix memory."""
+    sizes = {
+        # width, layers, heads, head size, dense ff, scan's inner width / state / dt rank / taps, chunk, vocabulary
+        "2b": (2048, 8, 16, 128, 8192, 4096, 16, 128, 4, 1024, 32000),
+        "7b": (4096, 8, 32, 128, 14336, 8192, 16, 256, 4, 1024, 32000),
+    }[name]
+    W, L, H, d, ff, inner, state, rank, taps, chunk, V = sizes
+    scan = {"type": "mamba1", "mixer": {"inner": inner, "state": state, "dt_rank": rank, "conv": taps}, "mlp": None}
+    att = {"type": "attention", "mixer": {
+        "heads": H, "kv_heads": max(1, H // 4), "dim": d, "vdim": d, "scale": d ** -0.5, "mask": {"size": chunk},
+        "rot": {"base": 500000.0, "dims": d // 2, "scaling": {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 8192}}},
+        "mlp": {"kind": "dense", "ff": ff}}
+    par = {"type": "parallel", "mixer": {
+        "left": {"heads": H, "kv_heads": max(1, H // 4), "dim": d // 2, "vdim": d // 2, "scale": (d // 2) ** -0.5,
+                 "conv": taps, "q_temp": {"coef": 0.5, "every": 1024}},
+        "right": {"heads": max(1, H // 2), "dim": d, "vdim": d, "gate_cap": 15.0}}, "mlp": {"kind": "dense", "ff": ff}}
+    layers = [(scan, att, scan, par)[i % 4] for i in range(L)]
+    nire = {"architecture": "Niresun", "vocab": V, "width": W, "norm": {"eps": 1e-5}, "layers": layers,
+            "max_position_embeddings": 8192, "torch_dtype": "bfloat16"}
+    llama = dict(LLAMA3_8B, vocab_size=V, hidden_size=W, intermediate_size=ff, num_hidden_layers=L,
+                 num_attention_heads=H, num_key_value_heads=max(1, H // 4), head_dim=d, bos_token_id=1, eos_token_id=2)
+    return nire, llama
+
+
 def takosun_run(args):
     """``--workload takosun``: prefill and decode of a Takosun model beside the Llama model of equal size; one JSON
     line. Decode: ``--steps`` steps at batch 1, 8 and 64 after 512-token prompts; prefill: one request of 512 and of
     2,048 tokens."""
+    beside_llama_run(args, "takosun", args.takosun_sizes, takosun_shapes(args.takosun_sizes))
+
+
+def niresun_run(args):
+    """``--workload niresun``: the same for a Niresun model."""
+    beside_llama_run(args, "niresun", args.niresun_sizes, niresun_shapes(args.niresun_sizes))
+
+
+def beside_llama_run(args, design, sizes, shapes):
     import gc
     import torch
-    out = {"metric": "takosun_beside_llama", "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
-           "steps": args.steps, "warmup": args.warmup, "config": {"sizes": args.takosun_sizes}, "models": {}}
-    for name, cfg in zip(("takosun", "llama"), takosun_shapes(args.takosun_sizes)):
+    out = {"metric": "%s_beside_llama" % design, "unit": "tokens/s", "n_gpus": 1, "dtype": args.dtype, "data": "synthetic",
+           "steps": args.steps, "warmup": args.warmup, "config": {"sizes": sizes}, "models": {}}
+    for name, cfg in zip((design, "llama"), shapes):
         engine = make_engine(cfg, args, max_num_seqs=64, dtype=args.dtype)
         m = {"weight_gb": round(weight_bytes(engine) / 1e9, 3),
              "decode_graphs": bool(engine.core.executor.use_graphs), "step_program": engine.core.executor.program is not None}
@@ -458,8 +494,8 @@ def takosun_run(args):
         del engine
         gc.collect()
         torch.cuda.empty_cache()
-    t, l = out["models"]["takosun"], out["models"]["llama"]
-    out["takosun_over_llama"] = {k: round(t[k] / l[k], 3) for k in t if k.endswith("tok_s")}
+    t, l = out["models"][design], out["models"]["llama"]
+    out["%s_over_llama" % design] = {k: round(t[k] / l[k], 3) for k in t if k.endswith("tok_s")}
     out["value"], out["higher_is_better"] = t["decode_b8_tok_s"], True
     print(json.dumps(out))
 
@@ -487,12 +523,14 @@ def main():
     ap.add_argument("--max-num-batched-tokens", type=int, default=8192)
     ap.add_argument("--gpu-memory-utilization", type=float, default=0.85)
     ap.add_argument("--skip-points", action="store_true", help="leave out the batch 1 and batch 64 runs")
-    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products", "takosun"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "serve", "products", "takosun", "niresun"],
                     help="decode: the default line (Llama-3-8B shape); serve: continuous batching of 64 requests at "
                          "Llama-2-7B shape, a line of its own; products: a layer's matrix products alone, the "
                          "library's against the engine's choice, at --rows; takosun: a Takosun model beside the Llama model "
                          "of equal size, prefill and decode")
     ap.add_argument("--takosun-sizes", default="2b", choices=["2b", "7b"], help="takosun: the layers' sizes")
+    ap.add_argument("--niresun-sizes", default="2b", choices=["2b", "7b"],
+                    help="niresun: the layers' sizes (a Niresun model beside the Llama model of equal size)")
     ap.add_argument("--rows", default="17,64,100,128,129,192,256,512,2048", help="products: numbers of rows")
     ap.add_argument("--prefill-chunk-size", type=int, default=1024, help="serve: longest portion of a prompt in a step")
     ap.add_argument("--shape", default="llama3-8b", choices=sorted(SHAPES),
@@ -530,6 +568,9 @@ def main():
         return
     if args.workload == "takosun":
         takosun_run(args)
+        return
+    if args.workload == "niresun":
+        niresun_run(args)
         return
     import torch
     shape_name, shape_cfg = SHAPES[args.shape]

@@ -848,11 +848,48 @@ class HipOps:
         self._state_view(state, inner * n, "selective_scan")
         _, seg_starts, slots, S = self._segments(batch, N)
         y = torch.empty((N, inner), dtype=x.dtype, device=x.device)
+        # segments longer than a chunk (portions of prompts) are cut into chunks that run side by side; which
+        # segments, and where their chunks' summaries lie, is worked out once a step on the host
+        chunk, max_chunks, bases, scratch = self.scan_chunk_tokens, 1, None, None
+        plan = self._chunk_plan(batch, chunk)
+        if plan is not None:
+            bases, entries, max_chunks = plan
+            scratch = torch.empty(entries * self.lib.lmsf_selective_scan_entry_floats(inner, n), dtype=torch.float32,
+                                  device=x.device)
         self._check(self.lib.lmsf_selective_scan(
             _ptr(x), _code(x.dtype), x.stride(0), _ptr(dt), dt.stride(0), _ptr(bc), bc.stride(0), int(b_at), int(c_at),
             _ptr(z), z.stride(0), _ptr(a_log), _ptr(d_skip), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots),
-            _ptr(y), y.stride(0), N, S, inner, n, self._stream()))
+            _ptr(y), y.stride(0), N, S, inner, n, int(chunk), int(max_chunks), _ptr(bases), _ptr(scratch), self._stream()))
         return y
+
+    scan_chunk_tokens = 64         # tokens of a chunk of the selective scan's chunked form
+    recurrent_chunked_min_tokens = 16   # segments from this many tokens on go to the matrix memory's chunked form
+    recurrent_parallel_min_chunks = 3   # and from this many chunks on the chunks run side by side
+
+    def _chunk_plan(self, batch, chunk: int):
+        """(per segment its first entry of scratch or -1, entries in all, the most chunks of a segment) for a step
+        that has segments longer than ``chunk`` tokens; None for a step without (and for a captured step, where
+        nothing may hang on the host's view of the segments: those are steps of single tokens)."""
+        if getattr(batch, "replayed", False) or getattr(batch, "all_single", False):
+            return None
+        key = ("chunk_plan", chunk)
+        aux = getattr(batch, "aux", None)
+        if aux is not None and key in aux:
+            return aux[key]
+        lens = getattr(batch, "host_seg_lens", None)
+        plan = None
+        if lens and max(lens) > chunk:
+            bases, at, most = [], 0, 1
+            for n in lens:
+                c = -(-n // chunk)
+                bases.append(at if c > 1 else -1)
+                if c > 1:
+                    at += c
+                    most = max(most, c)
+            plan = (self.upload_ints(bases, batch.seg_starts.device), at, most)
+        if aux is not None:
+            aux[key] = plan
+        return plan
 
     def mlstm_state_floats(self, heads: int, dim: int, vdim: int) -> int:
         return int(self.lib.lmsf_mlstm_state_floats(heads, dim, vdim))
@@ -880,6 +917,32 @@ class HipOps:
         self._state_view(state, self.mlstm_state_floats(heads, dim, vdim), "mlstm")
         _, seg_starts, slots, S = self._segments(batch, N)
         out = torch.empty((N, heads * vdim), dtype=q.dtype, device=q.device)
+        lens = getattr(batch, "host_seg_lens", None)
+        if not getattr(batch, "replayed", False) and not getattr(batch, "all_single", False) and lens \
+                and max(lens) >= self.recurrent_chunked_min_tokens:
+            # portions of prompts: chunks of tokens at a time (csrc/recurrent.hip: mlstm_chunk_kernel)
+            raw = torch.empty(self.lib.lmsf_mlstm_chunk_scratch_floats(N, heads, vdim), dtype=torch.float32, device=q.device)
+            # with segments of several chunks the chunks run side by side (three launches); their summaries and first
+            # states lie in scratch, a segment's chunks one behind the other
+            L = self.lib.lmsf_mlstm_chunk_tokens(int(dim))
+            bases = entries = None
+            n_entries, most = 0, 1
+            if L > 0 and max(lens) >= self.recurrent_parallel_min_chunks * L:
+                key = ("mlstm_chunks", L)
+                plan = batch.aux.get(key)
+                if plan is None:
+                    counts = [-(-n // L) for n in lens]
+                    firsts = [sum(counts[:i]) for i in range(len(counts))]
+                    plan = batch.aux[key] = (self.upload_ints(firsts, q.device), sum(counts), max(counts))
+                bases, n_entries, most = plan
+                entries = torch.empty(n_entries * self.lib.lmsf_mlstm_chunk_entry_floats(heads, dim, vdim),
+                                      dtype=torch.float32, device=q.device)
+            self._check(self.lib.lmsf_mlstm_chunked(
+                _ptr(q), _ptr(k), _ptr(v), _code(q.dtype), q.stride(0), _ptr(gates), gates.stride(0), _ptr(out_gate),
+                out_gate.stride(0), _ptr(norm_weight), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots),
+                _ptr(out), out.stride(0), _ptr(raw), N, S, int(heads), int(dim), int(vdim), float(q_scale),
+                float(gate_cap), float(eps), _ptr(bases), int(most), int(n_entries), _ptr(entries), self._stream()))
+            return out
         self._check(self.lib.lmsf_mlstm(
             _ptr(q), _ptr(k), _ptr(v), _code(q.dtype), q.stride(0), _ptr(gates), gates.stride(0), _ptr(out_gate),
             out_gate.stride(0), _ptr(norm_weight), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots), _ptr(out),

@@ -55,7 +55,14 @@ _SIGNATURES = {
     "lmsf_short_conv": (c_int, [_P, c_int, c_long, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, c_long, c_int, c_int, c_int,
                                 c_int, _P]),
     "lmsf_selective_scan": (c_int, [_P, c_int, c_long, _P, c_long, _P, c_long, c_int, c_int, _P, c_long, _P, _P, _P,
-                                    c_long, _P, _P, _P, c_long, c_int, c_int, c_int, c_int, _P]),
+                                    c_long, _P, _P, _P, c_long, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, _P]),
+    "lmsf_selective_scan_entry_floats": (c_long, [c_int, c_int]),
+    "lmsf_mlstm_chunk_scratch_floats": (c_long, [c_int, c_int, c_int]),
+    "lmsf_mlstm_chunked": (c_int, [_P, _P, _P, c_int, c_long, _P, c_long, _P, c_long, _P, _P, c_long, _P, _P, _P, c_long,
+                                   _P, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, _P, c_int, c_long,
+                                   _P, _P]),
+    "lmsf_mlstm_chunk_tokens": (c_int, [c_int]),
+    "lmsf_mlstm_chunk_entry_floats": (c_long, [c_int, c_int, c_int]),
     "lmsf_mlstm_state_floats": (c_long, [c_int, c_int, c_int]),
     "lmsf_mlstm": (c_int, [_P, _P, _P, c_int, c_long, _P, c_long, _P, c_long, _P, _P, c_long, _P, _P, _P, c_long, c_int,
                            c_int, c_int, c_int, c_int, c_float, c_float, c_float, _P]),

@@ -445,156 +445,11 @@ extern "C" int lmsf_selective_scan(const void* x, int dtype, long x_stride, cons
 //   out = o / rms(o) * w * sigmoid(g)      (rms over the head's dv entries, eps inside the root)
 // n is kept as one more column of S (a value entry that is always 1), so that n . q comes out of the same sums as
 // S^T q. The state of a slot: S and n as [H, d, dv + 1], then m as [H].
-// A workgroup: one head of one segment; thread (rg, vv) owns column vv of the rows rg, rg + RG, ... (RPT of them).
-template <typename T, int RPT>
-__global__ __launch_bounds__(256) void mlstm_kernel(
-    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, long qkv_stride,
-    const float* __restrict__ gates, long gates_stride, const T* __restrict__ og, long og_stride,
-    const float* __restrict__ norm_w, float* __restrict__ state, long state_stride, const int* __restrict__ seg_starts,
-    const int* __restrict__ state_slots, T* __restrict__ out, long out_stride, int H, int d, int dv, int VB,
-    float qscale, float cap, float eps, int TT) {
-  extern __shared__ float lds[];
-  const int RG = 256 / VB, dpad = RPT * RG, cols = dv + 1;
-  float* sq = lds;                   // [TT][dpad], zeros behind d
-  float* sk = sq + TT * dpad;        // [TT][dpad]
-  float* sv = sk + TT * dpad;        // [TT][VB]: v, then 1, then zeros
-  float* sg = sv + TT * VB;          // [TT][2]: i, f
-  float* so = sg + TT * 2;           // [TT][dv]
-  float* red = so + TT * dv;         // [RG][VB]
-  float* oext = red + RG * VB;       // [VB]
-  const int tid = threadIdx.x, vv = tid % VB, rg = tid / VB;
-  const int h = blockIdx.x, s = blockIdx.y;
-  const int start = seg_starts[s], end = seg_starts[s + 1];
-  float* st = state + (long)state_slots[s] * state_stride;
-  float* sS = st + (long)h * d * cols;
-  float* sm = st + (long)H * d * cols + h;
-  float S[RPT];
-#pragma unroll
-  for (int r = 0; r < RPT; ++r) {
-    const int dd = rg + r * RG;
-    S[r] = (dd < d && vv < cols) ? sS[(long)dd * cols + vv] : 0.f;
-  }
-  float m = sm[0];
-  for (int t0 = start; t0 < end; t0 += TT) {
-    const int nt = min(TT, end - t0);
-    for (int i = tid; i < nt * dpad; i += 256) {
-      const int tt = i / dpad, dd = i % dpad;
-      const long t = t0 + tt;
-      sq[i] = dd < d ? to_f32<T>(q[t * qkv_stride + h * d + dd]) * qscale : 0.f;
-      sk[i] = dd < d ? to_f32<T>(k[t * qkv_stride + h * d + dd]) : 0.f;
-    }
-    for (int i = tid; i < nt * VB; i += 256) {
-      const int tt = i / VB, e = i % VB;
-      sv[i] = e < dv ? to_f32<T>(v[(long)(t0 + tt) * qkv_stride + h * dv + e]) : e == dv ? 1.f : 0.f;
-    }
-    for (int tt = tid; tt < nt; tt += 256) {
-      const float ip = gates[(long)(t0 + tt) * gates_stride + h], fp = gates[(long)(t0 + tt) * gates_stride + H + h];
-      sg[tt * 2] = cap * tanhf(ip / cap);
-      sg[tt * 2 + 1] = rc_logsigmoid(cap * tanhf(fp / cap));
-    }
-    __syncthreads();
-    for (int tt = 0; tt < nt; ++tt) {
-      const float gi = sg[tt * 2], gf = sg[tt * 2 + 1];
-      const float m_new = fmaxf(gf + m, gi);
-      const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
-      m = m_new;
-      const float tv = take * sv[tt * VB + vv];
-      float acc = 0.f;
-#pragma unroll
-      for (int r = 0; r < RPT; ++r) {
-        const int dd = rg + r * RG;
-        S[r] = keep * S[r] + sk[tt * dpad + dd] * tv;
-        acc += S[r] * sq[tt * dpad + dd];
-      }
-      if (RG > 1) {
-        red[rg * VB + vv] = acc;
-        __syncthreads();
-        if (rg == 0) {
-          float total = 0.f;
-          for (int g = 0; g < RG; ++g) total += red[g * VB + vv];
-          oext[vv] = total;
-        }
-      } else {
-        oext[vv] = acc;
-      }
-      __syncthreads();
-      if (tid < dv) so[tt * dv + tid] = oext[tid] / (fmaxf(fabsf(oext[dv]), expf(-m)) + 1e-6f);
-      __syncthreads();
-    }
-    // the heads' norm, the weight and the output gate, a wave a token
-    for (int tt = tid / LMSF_WAVE; tt < nt; tt += 256 / LMSF_WAVE) {
-      const int lane = tid % LMSF_WAVE;
-      float ss = 0.f;
-      for (int e = lane; e < dv; e += LMSF_WAVE) ss += so[tt * dv + e] * so[tt * dv + e];
-      ss = wave_sum(ss);
-      const float inv = 1.f / sqrtf(ss / (float)dv + eps);
-      const long t = t0 + tt;
-      for (int e = lane; e < dv; e += LMSF_WAVE) {
-        const float g = to_f32<T>(og[t * og_stride + h * dv + e]);
-        out[t * out_stride + h * dv + e] = from_f32<T>(so[tt * dv + e] * inv * norm_w[h * dv + e] * rc_sigmoid(g));
-      }
-    }
-    __syncthreads();
-  }
-#pragma unroll
-  for (int r = 0; r < RPT; ++r) {
-    const int dd = rg + r * RG;
-    if (dd < d && vv < cols) sS[(long)dd * cols + vv] = S[r];
-  }
-  if (tid == 0) sm[0] = m;
-}
+// Three forms follow: chunks of a segment one after the other or side by side (portions of prompts), and token by
+// token with the memory streamed once (steps of single tokens).
 
 // floats of state a slot needs: S and n as [H, d, dv + 1], m as [H]
 extern "C" long lmsf_mlstm_state_floats(int H, int d, int dv) { return (long)H * d * (dv + 1) + H; }
-
-extern "C" int lmsf_mlstm(const void* q, const void* k, const void* v, int dtype, long qkv_stride, const float* gates,
-                          long gates_stride, const void* og, long og_stride, const float* norm_w, float* state,
-                          long state_stride, const int* seg_starts, const int* state_slots, void* out, long out_stride,
-                          int n_tokens, int n_segments, int H, int d, int dv, float qscale, float cap, float eps,
-                          hipStream_t stream) {
-  LMSF_CHECK(q && k && v && gates && og && norm_w && state && seg_starts && state_slots && out, "mlstm: null pointer");
-  LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "mlstm: unknown dtype code %d", dtype);
-  LMSF_CHECK(H > 0 && H <= 65535 && d > 0 && dv > 0 && dv <= 255, "mlstm: bad sizes H=%d d=%d dv=%d (dv <= 255)", H, d, dv);
-  LMSF_CHECK(cap > 0.f, "mlstm: the gates' cap must be > 0");
-  LMSF_CHECK(gates_stride >= 2 * H && og_stride >= (long)H * dv && out_stride >= (long)H * dv &&
-                 state_stride >= lmsf_mlstm_state_floats(H, d, dv),
-             "mlstm: strides too small");
-  LMSF_CHECK(n_tokens >= 0 && n_segments >= 0 && n_segments <= 65535, "mlstm: bad counts");
-  if (n_tokens == 0 || n_segments == 0) return 0;
-  int VB = 16;
-  while (VB < dv + 1) VB *= 2;
-  const int RG = 256 / VB;
-  const int rows = (d + RG - 1) / RG;
-  LMSF_CHECK(rows <= 128, "mlstm: a head of %d x %d does not fit a workgroup's registers", d, dv);
-  const int RPT = rows <= 4 ? 4 : rows <= 8 ? 8 : rows <= 16 ? 16 : rows <= 32 ? 32 : rows <= 64 ? 64 : 128;
-  const int dpad = RPT * RG;
-  int TT = 16;
-  size_t smem = 0;
-  for (;; TT /= 2) {
-    smem = ((size_t)TT * (2 * dpad + VB + 2 + dv) + (size_t)RG * VB + VB) * sizeof(float);
-    if (smem <= 60 * 1024 || TT == 1) break;
-  }
-  LMSF_CHECK(smem <= 64 * 1024, "mlstm: a head of %d x %d needs %zu bytes of LDS", d, dv, smem);
-  dim3 grid(H, n_segments), block(256);
-#define ML(T, R)                                                                                                       \
-  hipLaunchKernelGGL((mlstm_kernel<T, R>), grid, block, smem, stream, (const T*)q, (const T*)k, (const T*)v,           \
-                     qkv_stride, gates, gates_stride, (const T*)og, og_stride, norm_w, state, state_stride, seg_starts, \
-                     state_slots, (T*)out, out_stride, H, d, dv, VB, qscale, cap, eps, TT)
-#define ML_T(T)                          \
-  do {                                   \
-    if (RPT == 4) ML(T, 4);              \
-    else if (RPT == 8) ML(T, 8);         \
-    else if (RPT == 16) ML(T, 16);       \
-    else if (RPT == 32) ML(T, 32);       \
-    else if (RPT == 64) ML(T, 64);       \
-    else ML(T, 128);                     \
-  } while (0)
-  if (dtype == LMSF_F32) ML_T(float); else ML_T(bf16_t);
-#undef ML_T
-#undef ML
-  LMSF_LAUNCH_CHECK("mlstm");
-  return 0;
-}
 
 // ---------------------------------------------------------------- the matrix memory over chunks of tokens
 // The same recurrence for segments of many tokens, a chunk of L tokens at a time. With F_t the sum of the log forget
@@ -602,10 +457,10 @@ extern "C" int lmsf_mlstm(const void* q, const void* k, const void* v, int dtype
 // before the chunk), the running maximum is m_t = F_t + M_t and
 //   S_t = exp(m_0 - M_t) S_0 + sum_{s <= t} exp(g_s - M_t) k_s v_s^T        (every weight <= 1)
 // so that a chunk is three small matrix products: P = (Q K^T) * exp(g_s - M_t) below the diagonal, [O | n.q] = w_0 Q
-// [S_0 | n_0] + P [V | 1], and the chunk's last S from K^T (w [V | 1]). A workgroup of 1,024 threads (four waves a SIMD
+// [S_0 | n_0] + P [V | 1], and the chunk's last S from K^T (w [V | 1]); O and max(|n.q|, exp(-m_t)) + 1e-6 are left
+// in float32 for the kernel that divides and norms the heads. A workgroup of 1,024 threads (four waves a SIMD
 // hide one another's waits for LDS): one head of one segment and a block of DVB value columns (n is carried as one more
-// column, as in the token-by-token form); chunks one after the other, a thread an entry of each product.
-// o = O / (max(|n.q|, exp(-m_t)) + 1e-6) is left in float32 for the kernel that norms the heads.
+// column, by the first block); chunks one after the other, a thread an entry of each product.
 #define MLC_THREADS 1024
 
 // MODE 0: a segment's chunks one after the other in one workgroup, the state from the slot and back to it.
@@ -620,7 +475,7 @@ __global__ __launch_bounds__(MLC_THREADS) void mlstm_chunk_kernel(
     const float* __restrict__ gates, long gates_stride, float* __restrict__ state, long state_stride,
     const int* __restrict__ seg_starts, const int* __restrict__ state_slots, float* __restrict__ o_raw, long o_stride,
     int H, int d, int dv, int L, int DVB, float qscale, float cap, int n_vb, const int* __restrict__ chunk_base,
-    float* __restrict__ sc_U, float* __restrict__ sc_fg, float* __restrict__ sc_m0) {
+    float* __restrict__ sc_U, float* __restrict__ sc_fg, float* __restrict__ sc_m0, float* __restrict__ den) {
   extern __shared__ float lds[];
   // row lengths in LDS are odd, so that threads that walk down neighbouring rows meet different banks
   const int dp = d | 1, NCp = (DVB + 1) | 1, Lp = L | 1;
@@ -638,7 +493,9 @@ __global__ __launch_bounds__(MLC_THREADS) void mlstm_chunk_kernel(
   const int h = blockIdx.x, s = blockIdx.y;
   const int vb = MODE == 0 ? blockIdx.z : blockIdx.z % n_vb, j = MODE == 0 ? 0 : blockIdx.z / n_vb;
   const int e0 = vb * DVB;
-  const int nb = min(DVB, dv - e0), cols = dv + 1, NC = nb + 1;
+  // (n is carried by the first block of columns alone: it is that block's to read and to write, and the other blocks
+  // need nothing of it, because the division by max(|n . q|, exp(-m)) + 1e-6 is left to the kernel that follows)
+  const int nb = min(DVB, dv - e0), cols = dv + 1, NC = nb + (vb == 0 ? 1 : 0);
   const int seg_start = seg_starts[s], seg_end = seg_starts[s + 1];
   if (MODE != 0 && j * L >= seg_end - seg_start) return;
   const int start = MODE == 0 ? seg_start : seg_start + j * L;
@@ -727,9 +584,10 @@ __global__ __launch_bounds__(MLC_THREADS) void mlstm_chunk_kernel(
       __syncthreads();
       for (int i = tid; i < nt * nb; i += MLC_THREADS) {
         const int t = i / nb, c = i % nb;
-        const float den = fmaxf(fabsf(so[t * NCp + nb]), expf(-(sF[t] + sM[t]))) + 1e-6f;
-        o_raw[(long)(t0 + t) * o_stride + h * dv + e0 + c] = so[t * NCp + c] / den;
+        o_raw[(long)(t0 + t) * o_stride + h * dv + e0 + c] = so[t * NCp + c];
       }
+      if (vb == 0 && tid < nt)
+        den[(long)(t0 + tid) * H + h] = fmaxf(fabsf(so[tid * NCp + nb]), expf(-(sF[tid] + sM[tid]))) + 1e-6f;
     } else {
       __syncthreads();
     }
@@ -804,9 +662,10 @@ __global__ __launch_bounds__(256) void mlstm_fold_kernel(float* __restrict__ sta
   st[(long)h * per + i] = S;       // (the slot's m is written by the last chunk's workgroup of the launch that follows:
 }                                  // here other workgroups of the head may not have read it yet)
 
-// out[t, h, e] = o[t, h, e] / rms_e(o[t, h, :]) * w[h, e] * sigmoid(g[t, h, e]); a wave a (token, head)
+// o = num / den[t, h];  out[t, h, e] = o[e] / rms_e(o) * w[h, e] * sigmoid(g[t, h, e]); a wave a (token, head)
 template <typename T>
 __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __restrict__ o, long o_stride,
+                                                             const float* __restrict__ den,
                                                              const T* __restrict__ og, long og_stride,
                                                              const float* __restrict__ w, T* __restrict__ out,
                                                              long out_stride, int n_tokens, int H, int dv, float eps) {
@@ -815,18 +674,96 @@ __global__ __launch_bounds__(256) void head_norm_gate_kernel(const float* __rest
   const long t = unit / H;
   const int h = unit % H, lane = threadIdx.x % LMSF_WAVE;
   const float* row = o + t * o_stride + (long)h * dv;
+  const float by = 1.f / den[t * H + h];
   float ss = 0.f;
-  for (int e = lane; e < dv; e += LMSF_WAVE) ss += row[e] * row[e];
+  for (int e = lane; e < dv; e += LMSF_WAVE) ss += (row[e] * by) * (row[e] * by);
   ss = wave_sum(ss);
-  const float inv = 1.f / sqrtf(ss / (float)dv + eps);
+  const float inv = by / sqrtf(ss / (float)dv + eps);
   for (int e = lane; e < dv; e += LMSF_WAVE) {
     const float g = to_f32<T>(og[t * og_stride + (long)h * dv + e]);
     out[t * out_stride + (long)h * dv + e] = from_f32<T>(row[e] * inv * w[h * dv + e] * rc_sigmoid(g));
   }
 }
 
-// the chunked form's temporary: float32 [n_tokens, H * dv]
-extern "C" long lmsf_mlstm_chunk_scratch_floats(int n_tokens, int H, int dv) { return (long)n_tokens * H * dv; }
+// The matrix memory for steps of single tokens, where a step is one pass over every request's state and nothing but
+// memory counts: a workgroup takes one head of one segment and 64 of its value columns (the first block n as well);
+// wave w walks the rows w, w + 4, ..., a lane a column, so that every load of S is 256 consecutive bytes, eight rows
+// asked for at a time. S^T q and max(|n . q|, exp(-m)) + 1e-6 are left in float32 for the kernel that divides and
+// norms the heads. Segments of more than one token are walked token by token (correct, not fast).
+#define MLD_COLS 64
+
+template <typename T>
+__global__ __launch_bounds__(256) void mlstm_token_kernel(
+    const T* __restrict__ q, const T* __restrict__ k, const T* __restrict__ v, long qkv_stride,
+    const float* __restrict__ gates, long gates_stride, float* __restrict__ state, long state_stride,
+    const int* __restrict__ seg_starts, const int* __restrict__ state_slots, float* __restrict__ o_raw, long o_stride,
+    float* __restrict__ den, int H, int d, int dv, float qscale, float cap) {
+  extern __shared__ float lds[];
+  float* sq = lds;               // [d]
+  float* sk = sq + d;            // [d]
+  float* so = sk + d;            // [4][64]
+  const int tid = threadIdx.x, wave = tid / LMSF_WAVE, lane = tid % LMSF_WAVE;
+  const int h = blockIdx.x, s = blockIdx.y, e0 = blockIdx.z * MLD_COLS;
+  const int cols = dv + 1;
+  const bool col_ok = e0 + lane < dv;
+  float* st = state + (long)state_slots[s] * state_stride;
+  float* gS = st + (long)h * d * cols;
+  float* gm = st + (long)H * d * cols + h;
+  float m = gm[0];
+  for (int t = seg_starts[s]; t < seg_starts[s + 1]; ++t) {
+    __syncthreads();
+    for (int i = tid; i < d; i += 256) {
+      sq[i] = to_f32<T>(q[(long)t * qkv_stride + h * d + i]) * qscale;
+      sk[i] = to_f32<T>(k[(long)t * qkv_stride + h * d + i]);
+    }
+    const float vv = col_ok ? to_f32<T>(v[(long)t * qkv_stride + h * dv + e0 + lane]) : 0.f;
+    const float gi = cap * tanhf(gates[(long)t * gates_stride + h] / cap);
+    const float gf = rc_logsigmoid(cap * tanhf(gates[(long)t * gates_stride + H + h] / cap));
+    const float m_new = fmaxf(gf + m, gi);
+    const float keep = expf(gf + m - m_new), take = expf(gi - m_new);
+    m = m_new;
+    __syncthreads();
+    float acc = 0.f;
+    for (int d0 = wave; d0 < d; d0 += 4 * 8) {
+      float r[8];
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int dd = d0 + 4 * j;
+        r[j] = (dd < d && col_ok) ? gS[(long)dd * cols + e0 + lane] : 0.f;
+      }
+#pragma unroll
+      for (int j = 0; j < 8; ++j) {
+        const int dd = d0 + 4 * j;
+        if (dd < d && col_ok) {
+          const float x = keep * r[j] + take * sk[dd] * vv;
+          gS[(long)dd * cols + e0 + lane] = x;
+          acc += x * sq[dd];
+        }
+      }
+    }
+    so[wave * MLD_COLS + lane] = acc;
+    if (wave == 1 && blockIdx.z == 0) {
+      // n and n . q, by the first block of columns alone: a lane a row
+      float part = 0.f;
+      for (int dd = lane; dd < d; dd += LMSF_WAVE) {
+        const float x = keep * gS[(long)dd * cols + dv] + take * sk[dd];
+        gS[(long)dd * cols + dv] = x;
+        part += x * sq[dd];
+      }
+      part = wave_sum(part);
+      if (lane == 0) den[(long)t * H + h] = fmaxf(fabsf(part), expf(-m)) + 1e-6f;
+    }
+    __syncthreads();
+    if (wave == 0 && col_ok)
+      o_raw[(long)t * o_stride + h * dv + e0 + lane] =
+          so[lane] + so[MLD_COLS + lane] + so[2 * MLD_COLS + lane] + so[3 * MLD_COLS + lane];
+  }
+  if (tid == 0 && blockIdx.z == 0) gm[0] = m;
+}
+
+// the temporary of the forms that leave the division to the heads' kernel: numerators float32 [n_tokens, H * dv], then
+// denominators [n_tokens, H]
+extern "C" long lmsf_mlstm_chunk_scratch_floats(int n_tokens, int H, int dv) { return (long)n_tokens * H * (dv + 1); }
 
 // tokens of a chunk at heads of d (the most for which a workgroup's operands fit its LDS)
 extern "C" int lmsf_mlstm_chunk_tokens(int d) {
@@ -888,7 +825,7 @@ extern "C" int lmsf_mlstm_chunked(const void* q, const void* k, const void* v, i
     hipLaunchKernelGGL((mlstm_chunk_kernel<T, MODE>), GRID, dim3(MLC_THREADS), smem, stream, (const T*)q,          \
                        (const T*)k, (const T*)v, qkv_stride, gates, gates_stride, state, state_stride, seg_starts, \
                        state_slots, o_raw, (long)H * dv, H, d, dv, L, DVB, qscale, cap, n_vb, chunk_base, sc_U,    \
-                       sc_fg, sc_m0);                                                                              \
+                       sc_fg, sc_m0, o_raw + (long)n_tokens * H * dv);                                             \
   } while (0)
   float* sc_U = entries;
   float* sc_fg = entries ? entries + n_entries * H * d * (dv + 1) : nullptr;
@@ -913,11 +850,56 @@ extern "C" int lmsf_mlstm_chunked(const void* q, const void* k, const void* v, i
   const long units = (long)n_tokens * H;
   dim3 ngrid((unsigned)((units + 3) / 4)), block(256);
   if (dtype == LMSF_F32)
-    hipLaunchKernelGGL((head_norm_gate_kernel<float>), ngrid, block, 0, stream, o_raw, (long)H * dv, (const float*)og,
+    hipLaunchKernelGGL((head_norm_gate_kernel<float>), ngrid, block, 0, stream, o_raw, (long)H * dv,
+                       o_raw + (long)n_tokens * H * dv, (const float*)og,
                        og_stride, norm_w, (float*)out, out_stride, n_tokens, H, dv, eps);
   else
-    hipLaunchKernelGGL((head_norm_gate_kernel<bf16_t>), ngrid, block, 0, stream, o_raw, (long)H * dv, (const bf16_t*)og,
+    hipLaunchKernelGGL((head_norm_gate_kernel<bf16_t>), ngrid, block, 0, stream, o_raw, (long)H * dv,
+                       o_raw + (long)n_tokens * H * dv, (const bf16_t*)og,
                        og_stride, norm_w, (bf16_t*)out, out_stride, n_tokens, H, dv, eps);
+  LMSF_LAUNCH_CHECK("head_norm_gate");
+  return 0;
+}
+
+// The same function for steps of few tokens a segment (decoding): mlstm_token_kernel, then the heads' norm and gate.
+extern "C" int lmsf_mlstm_tokens(const void* q, const void* k, const void* v, int dtype, long qkv_stride,
+                                 const float* gates, long gates_stride, const void* og, long og_stride,
+                                 const float* norm_w, float* state, long state_stride, const int* seg_starts,
+                                 const int* state_slots, void* out, long out_stride, float* o_raw, int n_tokens,
+                                 int n_segments, int H, int d, int dv, float qscale, float cap, float eps,
+                                 hipStream_t stream) {
+  LMSF_CHECK(q && k && v && gates && og && norm_w && state && seg_starts && state_slots && out && o_raw,
+             "mlstm_tokens: null pointer");
+  LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "mlstm_tokens: unknown dtype code %d", dtype);
+  LMSF_CHECK(H > 0 && H <= 65535 && d > 0 && d <= 4096 && dv > 0, "mlstm_tokens: bad sizes H=%d d=%d dv=%d", H, d, dv);
+  LMSF_CHECK(cap > 0.f, "mlstm_tokens: the gates' cap must be > 0");
+  LMSF_CHECK(gates_stride >= 2 * H && og_stride >= (long)H * dv && out_stride >= (long)H * dv &&
+                 state_stride >= lmsf_mlstm_state_floats(H, d, dv),
+             "mlstm_tokens: strides too small");
+  LMSF_CHECK(n_tokens >= 0 && n_segments >= 0 && n_segments <= 65535 && (dv + MLD_COLS - 1) / MLD_COLS <= 65535,
+             "mlstm_tokens: bad counts");
+  if (n_tokens == 0 || n_segments == 0) return 0;
+  dim3 grid(H, n_segments, (dv + MLD_COLS - 1) / MLD_COLS), block(256);
+  const size_t smem = (size_t)(2 * d + 4 * MLD_COLS) * sizeof(float);
+  const long units = (long)n_tokens * H;
+  dim3 ngrid((unsigned)((units + 3) / 4));
+  if (dtype == LMSF_F32) {
+    hipLaunchKernelGGL((mlstm_token_kernel<float>), grid, block, smem, stream, (const float*)q, (const float*)k,
+                       (const float*)v, qkv_stride, gates, gates_stride, state, state_stride, seg_starts, state_slots,
+                       o_raw, (long)H * dv, o_raw + (long)n_tokens * H * dv, H, d, dv, qscale, cap);
+    LMSF_LAUNCH_CHECK("mlstm_tokens");
+    hipLaunchKernelGGL((head_norm_gate_kernel<float>), ngrid, block, 0, stream, o_raw, (long)H * dv,
+                       o_raw + (long)n_tokens * H * dv, (const float*)og,
+                       og_stride, norm_w, (float*)out, out_stride, n_tokens, H, dv, eps);
+  } else {
+    hipLaunchKernelGGL((mlstm_token_kernel<bf16_t>), grid, block, smem, stream, (const bf16_t*)q, (const bf16_t*)k,
+                       (const bf16_t*)v, qkv_stride, gates, gates_stride, state, state_stride, seg_starts, state_slots,
+                       o_raw, (long)H * dv, o_raw + (long)n_tokens * H * dv, H, d, dv, qscale, cap);
+    LMSF_LAUNCH_CHECK("mlstm_tokens");
+    hipLaunchKernelGGL((head_norm_gate_kernel<bf16_t>), ngrid, block, 0, stream, o_raw, (long)H * dv,
+                       o_raw + (long)n_tokens * H * dv, (const bf16_t*)og,
+                       og_stride, norm_w, (bf16_t*)out, out_stride, n_tokens, H, dv, eps);
+  }
   LMSF_LAUNCH_CHECK("head_norm_gate");
   return 0;
 }

@@ -943,10 +943,12 @@ class HipOps:
                 _ptr(out), out.stride(0), _ptr(raw), N, S, int(heads), int(dim), int(vdim), float(q_scale),
                 float(gate_cap), float(eps), _ptr(bases), int(most), int(n_entries), _ptr(entries), self._stream()))
             return out
-        self._check(self.lib.lmsf_mlstm(
+        # steps of single tokens, and of portions of a few: one pass over every request's state
+        raw = torch.empty(self.lib.lmsf_mlstm_chunk_scratch_floats(N, heads, vdim), dtype=torch.float32, device=q.device)
+        self._check(self.lib.lmsf_mlstm_tokens(
             _ptr(q), _ptr(k), _ptr(v), _code(q.dtype), q.stride(0), _ptr(gates), gates.stride(0), _ptr(out_gate),
             out_gate.stride(0), _ptr(norm_weight), _ptr(state), state.stride(0), _ptr(seg_starts), _ptr(slots), _ptr(out),
-            out.stride(0), N, S, int(heads), int(dim), int(vdim), float(q_scale), float(gate_cap), float(eps),
+            out.stride(0), _ptr(raw), N, S, int(heads), int(dim), int(vdim), float(q_scale), float(gate_cap), float(eps),
             self._stream()))
         return out
 

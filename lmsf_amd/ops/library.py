@@ -61,11 +61,11 @@ _SIGNATURES = {
     "lmsf_mlstm_chunked": (c_int, [_P, _P, _P, c_int, c_long, _P, c_long, _P, c_long, _P, _P, c_long, _P, _P, _P, c_long,
                                    _P, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, _P, c_int, c_long,
                                    _P, _P]),
+    "lmsf_mlstm_tokens": (c_int, [_P, _P, _P, c_int, c_long, _P, c_long, _P, c_long, _P, _P, c_long, _P, _P, _P, c_long, _P,
+                                  c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_float, _P]),
     "lmsf_mlstm_chunk_tokens": (c_int, [c_int]),
     "lmsf_mlstm_chunk_entry_floats": (c_long, [c_int, c_int, c_int]),
     "lmsf_mlstm_state_floats": (c_long, [c_int, c_int, c_int]),
-    "lmsf_mlstm": (c_int, [_P, _P, _P, c_int, c_long, _P, c_long, _P, c_long, _P, _P, c_long, _P, _P, _P, c_long, c_int,
-                           c_int, c_int, c_int, c_int, c_float, c_float, c_float, _P]),
     "lmsf_attn_prepare": (c_int, [_P, c_long, _P, c_long, _P, c_long, c_int, _P, _P, c_int, c_int, _P, _P, c_long, _P, _P,
                                   c_long, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_int, c_float, c_float, c_int,
                                   _P]),

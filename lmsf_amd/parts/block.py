@@ -28,7 +28,7 @@ class PreNormResidualBlock(Block):
         super().__init__(prefix, rt, mixer, feed_forward, norms)
         self.has_ffn = not getattr(feed_forward, "absent", False)
         if self.has_ffn and "post_mixer" not in norms:
-            raise ValueError("block %s needs the norm post_mixer before its feed-forward" % prefix)
+            raise ValueError("block %s needs norms post_mixer (before its feed-forward)" % type(self).__name__)
 
     @property
     def accepts_pending_branch(self) -> bool:

@@ -27,9 +27,15 @@ def ops():
     return get_ops()
 
 
-def check(got, ref, dtype, what=""):
+def check(got, ref, dtype, what="", model=None):
+    """``model`` = (configuration, weights, tokens): float32 then may differ by three times what float32 rounding
+    costs the plain implementation itself on these tokens, where that is more than TOL_F32 (a configuration whose
+    logits hang on small differences)."""
     if dtype == "float32":
-        assert rel_err(got, ref) < TOL_F32, (what, rel_err(got, ref))
+        tol = TOL_F32
+        if model is not None:
+            tol = max(tol, 3 * rel_err(plain_logits(model[0], model[1], model[2], dtype=torch.float32), ref))
+        assert rel_err(got, ref) < tol, (what, rel_err(got, ref), tol)
     else:
         # (rounding has outliers at positions whose logits hang on small differences: one position in fifty, or one,
         # may pass the limit, none three times the limit; a fault moves many rows, and by more)
@@ -256,12 +262,12 @@ def test_every_kind_of_layer_alone(tmp_path, which, index, dtype):
     V = cfg["vocab"]
     a, b = tokens(75, V, 1), tokens(30, V, 2)
     ref = {"a": plain_logits(cfg, w, a), "b": plain_logits(cfg, w, b)}
-    check(replay(core.executor, StepEntry, {"a": a}, [[("a", 75)]])["a"], ref["a"], dtype, "whole")
+    check(replay(core.executor, StepEntry, {"a": a}, [[("a", 75)]])["a"], ref["a"], dtype, "whole", (cfg, w, a))
     steps = [[("a", 7), ("b", 2)], [("a", 2)], [("b", 20), ("a", 33)], [("a", 1), ("b", 1)], [("a", 22), ("b", 1)]] + \
             [[("a", 1), ("b", 1)]] * 6 + [[("a", 1)]] * 4
     got = replay(core.executor, StepEntry, {"a": a, "b": b}, steps)
     for k in ref:
-        check(got[k], ref[k], dtype, k)
+        check(got[k], ref[k], dtype, k, (cfg, w, {"a": a, "b": b}[k]))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -285,7 +291,7 @@ def test_long_portions_take_the_forms_that_work_on_chunks(tmp_path, which, index
                 [[("a", 1)]] * 4
         got = replay(core.executor, StepEntry, {"a": a, "b": b}, steps)
         for k, t in (("a", a), ("b", b)):
-            check(got[k], plain_logits(cfg, w, t), dtype, k)
+            check(got[k], plain_logits(cfg, w, t), dtype, k, (cfg, w, t))
     finally:
         o.scan_chunk_tokens = keep
 
@@ -299,19 +305,20 @@ def test_four_ways_of_cutting_give_the_plain_logits(tmp_path, which, dtype):
     ex = core.executor
     a, b, c, d = tokens(150, V, 1), tokens(1, V, 2), tokens(67, V, 3), tokens(200, V, 4)
     ref = {k: plain_logits(cfg, w, t) for k, t in (("a", a), ("b", b), ("c", c), ("d", d))}
+    toks = {"a": a, "b": b, "c": c, "d": d}
     for k, t in (("a", a), ("b", b)):
-        check(replay(ex, StepEntry, {k: t}, [[(k, len(t))]])[k], ref[k], dtype, (k, "whole"))
+        check(replay(ex, StepEntry, {k: t}, [[(k, len(t))]])[k], ref[k], dtype, (k, "whole"), (cfg, w, t))
     got = replay(ex, StepEntry, {"a": a}, [[("a", 110)]] + [[("a", 1)]] * 40)["a"]
-    check(got, ref["a"], dtype, "decode")
+    check(got, ref["a"], dtype, "decode", (cfg, w, a))
     cuts = [15, 1, 2, 30, 16, 2, 33, 17, 19] + [1] * 15
     got = replay(ex, StepEntry, {"a": a}, [[("a", n)] for n in cuts])["a"]
-    check(got, ref["a"], dtype, "portions")
+    check(got, ref["a"], dtype, "portions", (cfg, w, a))
     # unequal requests together, three state slots for four requests; d starts in pages and a slot that were given back
     steps = [[("a", 64), ("b", 1), ("c", 3)], [("c", 2), ("a", 1)], [("a", 85), ("c", 61)], [("c", 1)],
              [("d", 2)], [("d", 197)], [("d", 1)]]
     got = replay(ex, StepEntry, {"a": a, "b": b, "c": c, "d": d}, steps)
     for k in ref:
-        check(got[k], ref[k], dtype, (k, "mixed"))
+        check(got[k], ref[k], dtype, (k, "mixed"), (cfg, w, toks[k]))
     core.storage.manager.check_invariants()
     assert core.storage.manager.num_free_pages(0) == 48 and core.storage.manager.num_free_state_slots() == 3
 
@@ -325,7 +332,7 @@ def test_sizes_at_which_the_matrix_core_kernels_run(tmp_path, dtype):
     steps = [[("a", 280)], [("a", 40), ("b", 60)]] + [[("a", 1), ("b", 1)]] * 10
     got = replay(core.executor, StepEntry, {"a": a, "b": b}, steps)
     for k, t in (("a", a), ("b", b)):
-        check(got[k], plain_logits(cfg, w, t), dtype, k)
+        check(got[k], plain_logits(cfg, w, t), dtype, k, (cfg, w, t))
 
 
 def peaked(cfg, seed, kind):
@@ -368,7 +375,7 @@ def test_keys_at_edges_and_far_away_decide(tmp_path, kind, dtype):
     if chunk:
         assert moved(first) > tol and moved(first - 1) < 1e-9          # the chunk's first key is seen, the one before is not
     got = replay(core.executor, StepEntry, {"a": t}, [[("a", 150)], [("a", 29)]] + [[("a", 1)]] * 8)["a"]
-    check(got, ref, dtype)
+    check(got, ref, dtype, "", (cfg, w, t))
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])
@@ -385,7 +392,7 @@ def test_long_decoding_from_graphs_equals_eager(tmp_path, dtype):
     ref = {"a": plain_logits(cfg, w, a), "b": plain_logits(cfg, w, b)}
     for k in ref:
         assert torch.equal(outs[0][k], outs[1][k]), k
-        check(outs[0][k], ref[k], dtype, k)
+        check(outs[0][k], ref[k], dtype, k, (cfg, w, {"a": a, "b": b}[k]))
 
 
 def test_greedy_generation_through_the_entry_point(tmp_path):

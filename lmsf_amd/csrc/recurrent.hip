@@ -80,6 +80,8 @@ extern "C" int lmsf_short_conv(const void* u, int dtype, long u_stride, const vo
   LMSF_CHECK((C + 255) / 256 <= 65535, "short_conv: too many channels");
   if (n_tokens == 0) return 0;
   dim3 grid(n_tokens, (C + 255) / 256), sgrid(n_segments, (C + 255) / 256), block(256);
+  // (a form with 16-byte accesses, a thread 8 neighbouring channels of a token, measured slower at 2,048 tokens of 4,096
+  // channels, 74 against 60 us, and at 8 tokens, 10.7 against 3.8: its weights' loads lie 64 bytes apart across a wave)
 #define SC(T, A)                                                                                                      \
   hipLaunchKernelGGL((short_conv_kernel<T, A>), grid, block, 0, stream, (const T*)u, u_stride, (const T*)w,           \
                      (const T*)bias, state, state_stride, seg_of, seg_starts, state_slots, (T*)out, out_stride, C, taps)

@@ -101,14 +101,16 @@ def test_gated_activation_in_the_tanh_form(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
-@pytest.mark.parametrize("C,taps,act", [(24, 3, None), (300, 4, "silu"), (8, 2, None), (40, 7, "silu"), (16, 1, None)])
-def test_short_convolution_over_cut_requests(dtype, C, taps, act):
+@pytest.mark.parametrize("C,taps,act,off", [(24, 3, None, 2), (300, 4, "silu", 2), (8, 2, None, 8), (40, 7, "silu", 8),
+                                            (16, 1, None, 2), (512, 4, "silu", 8), (72, 3, None, 8)])
+def test_short_convolution_over_cut_requests(dtype, C, taps, act, off):
     """Three requests; their tokens arrive in steps of unequal portions (down to one token, shorter than the filter),
-    in slots that do not follow their order; every output equals the convolution over the whole request."""
+    in slots that do not follow their order; every output equals the convolution over the whole request. The operand
+    is a view into wider rows, beginning on a 16-byte border (off 8) or not (off 2)."""
     o = ops()
     g = torch.Generator().manual_seed(C * taps)
     lens = {"a": 23, "b": 1, "c": 9}
-    u = {k: (torch.randn((n, C + 5), generator=g)).to(dtype) for k, n in lens.items()}
+    u = {k: (torch.randn((n, C + 16), generator=g)).to(dtype) for k, n in lens.items()}
     w = (torch.randn((C, taps), generator=g) * 0.5).to(dtype)
     bias = (torch.randn(C, generator=g) * 0.1).to(dtype) if act else None
     state = torch.zeros((4, C * max(taps - 1, 1) + 3), dtype=torch.float32, device="cuda")
@@ -117,7 +119,7 @@ def test_short_convolution_over_cut_requests(dtype, C, taps, act):
     at = {k: 0 for k in lens}
     got = {k: [] for k in lens}
     for step in steps:
-        x = torch.cat([u[k][at[k]:at[k] + n] for k, n in step]).cuda()[:, 2:2 + C]       # a view into wider rows
+        x = torch.cat([u[k][at[k]:at[k] + n] for k, n in step]).cuda()[:, off:off + C]   # a view into wider rows
         y = o.short_conv(x, w.cuda(), None if bias is None else bias.cuda(), state[:, 3:] if taps > 1 else None,
                          Step([n for _, n in step], [slot[k] for k, _ in step]), act)
         row = 0
@@ -126,7 +128,7 @@ def test_short_convolution_over_cut_requests(dtype, C, taps, act):
             row += n
             at[k] += n
     for k in lens:
-        ref = P.causal_conv(u[k][:, 2:2 + C].double(), w.double(), None if bias is None else bias.double())
+        ref = P.causal_conv(u[k][:, off:off + C].double(), w.double(), None if bias is None else bias.double())
         close(torch.cat(got[k]), P.silu(ref) if act else ref, dtype, scale=2.0)
     assert float(state[1].abs().max()) == 0.0 and float(state[:, :3].abs().max()) == 0.0     # nobody else's memory
 

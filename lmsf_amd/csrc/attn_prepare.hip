@@ -10,12 +10,14 @@
 
 #include <math.h>
 
+#include <algorithm>
+
 // Per token and head, in this order, each step optional:
 //   q, k <- x / sqrt(mean(x^2) + eps) over the head's dim entries                  (unit_norm)
 //   q, k <- rotation of the first ``rot`` entries, pairs (i, i + rot/2), by the position's angles (table != null)
 //   q    <- q (1 + temp_coef ln(floor((p + 1) / temp_every) + 1))                  (temp_every > 0)
 // q goes to q_out [N, H * D]; k to the token's slot of k_pages [pages, G, ps, D], v to v_pages [pages, G, D, ps]
-// (a negative slot stores nothing), all padded with zeros to D. A workgroup a token, a wave a head at a time.
+// (a negative slot stores nothing), all padded with zeros to D. A wave a (token, head).
 template <typename T>
 __global__ __launch_bounds__(256) void attn_prepare_kernel(
     const T* __restrict__ q, long q_stride, const T* __restrict__ k, long k_stride, const T* __restrict__ v,
@@ -31,7 +33,8 @@ __global__ __launch_bounds__(256) void attn_prepare_kernel(
   const float* cs = (table && p < max_pos) ? table + (long)p * rot : nullptr;
   const int half = rot / 2;
   const float temp = temp_every > 0 ? 1.f + temp_coef * logf((float)((p + 1) / temp_every) + 1.f) : 1.f;
-  for (int u = wave; u < H + 2 * G; u += 256 / LMSF_WAVE) {
+  // a wave a head of q, k or v: workgroup y takes the heads 4 y .. 4 y + 3 of the row q heads | k heads | v heads
+  for (int u = blockIdx.y * (256 / LMSF_WAVE) + wave; u < H + 2 * G; u += gridDim.y * (256 / LMSF_WAVE)) {
     if (u < H + G) {
       const bool is_q = u < H;
       const int head = is_q ? u : u - H;
@@ -93,13 +96,14 @@ extern "C" int lmsf_attn_prepare(const void* q, long q_stride, const void* k, lo
   LMSF_CHECK(!slots || (k_pages && v_pages && ps > 0 && num_pages > 0), "attn_prepare: slots without pages");
   LMSF_CHECK(temp_every >= 0, "attn_prepare: negative temperature period");
   if (n_tokens == 0) return 0;
+  const dim3 grid(n_tokens, std::min((H + 2 * G + 3) / 4, 65535));
   if (dtype == LMSF_F32)
-    hipLaunchKernelGGL((attn_prepare_kernel<float>), dim3(n_tokens), dim3(256), 0, stream, (const float*)q, q_stride,
+    hipLaunchKernelGGL((attn_prepare_kernel<float>), grid, dim3(256), 0, stream, (const float*)q, q_stride,
                        (const float*)k, k_stride, (const float*)v, v_stride, positions, table, rot, max_pos, slots,
                        (float*)q_out, qo_stride, (float*)k_pages, (float*)v_pages, H, G, dim, vdim, D, ps, unit_norm, eps,
                        temp_coef, temp_every);
   else
-    hipLaunchKernelGGL((attn_prepare_kernel<bf16_t>), dim3(n_tokens), dim3(256), 0, stream, (const bf16_t*)q, q_stride,
+    hipLaunchKernelGGL((attn_prepare_kernel<bf16_t>), grid, dim3(256), 0, stream, (const bf16_t*)q, q_stride,
                        (const bf16_t*)k, k_stride, (const bf16_t*)v, v_stride, positions, table, rot, max_pos, slots,
                        (bf16_t*)q_out, qo_stride, (bf16_t*)k_pages, (bf16_t*)v_pages, H, G, dim, vdim, D, ps, unit_norm,
                        eps, temp_coef, temp_every);

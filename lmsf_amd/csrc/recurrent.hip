@@ -24,25 +24,28 @@ __device__ __forceinline__ float rc_logsigmoid(float z) { return fminf(z, 0.f) -
 // ---------------------------------------------------------------- short causal convolution
 // out[t, c] = act(bias[c] + sum_j w[c, j] u[t - taps + 1 + j, c]); an input before the segment's first token is
 // the request's earlier input, kept in the state as [C, taps - 1] (oldest first; zeros before the request began).
-// ACT 0: none, 1: silu. The state is brought up to date by the second kernel, launched after the first.
+// ACT 0: none, 1: silu. The state is brought up to date by the second kernel, launched after the first; in a step of
+// single tokens (``single``) the thread of a (token, channel) is the only one that reads that channel's state, and
+// moves it on itself.
 template <typename T, int ACT>
 __global__ __launch_bounds__(256) void short_conv_kernel(const T* __restrict__ u, long u_stride, const T* __restrict__ w,
-                                                         const T* __restrict__ bias, const float* __restrict__ state,
+                                                         const T* __restrict__ bias, float* __restrict__ state,
                                                          long state_stride, const int* __restrict__ seg_of,
                                                          const int* __restrict__ seg_starts,
                                                          const int* __restrict__ state_slots, T* __restrict__ out,
-                                                         long out_stride, int C, int taps) {
+                                                         long out_stride, int C, int taps, int single) {
   const int t = blockIdx.x;
   const int c = blockIdx.y * 256 + threadIdx.x;
   if (c >= C) return;
   const int s = seg_of[t];
   const int start = seg_starts[s];
-  const float* st = state + (long)state_slots[s] * state_stride + (long)c * (taps - 1);
+  float* st = state + (long)state_slots[s] * state_stride + (long)c * (taps - 1);
   float acc = bias ? to_f32<T>(bias[c]) : 0.f;
   for (int j = 0; j < taps; ++j) {
     const int src = t - (taps - 1) + j;
     const float x = src >= start ? to_f32<T>(u[(long)src * u_stride + c]) : st[(taps - 1) + (src - start)];
     acc += to_f32<T>(w[(long)c * taps + j]) * x;
+    if (single && j > 0) st[j - 1] = x;          // (read above at j, written at j - 1: the state moves on by one token)
   }
   if (ACT == 1) acc = acc / (1.f + expf(-acc));
   out[(long)t * out_stride + c] = from_f32<T>(acc);
@@ -69,7 +72,7 @@ __global__ __launch_bounds__(256) void short_conv_state_kernel(const T* __restri
 extern "C" int lmsf_short_conv(const void* u, int dtype, long u_stride, const void* w, const void* bias, int act,
                                float* state, long state_stride, const int* seg_of, const int* seg_starts,
                                const int* state_slots, void* out, long out_stride, int n_tokens, int n_segments, int C,
-                               int taps, hipStream_t stream) {
+                               int taps, int single, hipStream_t stream) {
   LMSF_CHECK(u && w && out && seg_of && seg_starts && state_slots, "short_conv: null pointer");
   LMSF_CHECK(dtype == LMSF_F32 || dtype == LMSF_BF16, "short_conv: unknown dtype code %d", dtype);
   LMSF_CHECK(C > 0 && taps >= 1 && taps <= 64, "short_conv: bad sizes C=%d taps=%d", C, taps);
@@ -77,6 +80,7 @@ extern "C" int lmsf_short_conv(const void* u, int dtype, long u_stride, const vo
   LMSF_CHECK(u_stride >= C && out_stride >= C && state_stride >= (long)C * (taps - 1), "short_conv: strides too small");
   LMSF_CHECK(act == 0 || act == 1, "short_conv: unknown activation %d", act);
   LMSF_CHECK(n_tokens >= 0 && n_segments >= 0 && n_segments <= n_tokens, "short_conv: bad counts");
+  LMSF_CHECK(!single || n_segments == n_tokens, "short_conv: a step of single tokens has as many segments as tokens");
   LMSF_CHECK((C + 255) / 256 <= 65535, "short_conv: too many channels");
   if (n_tokens == 0) return 0;
   dim3 grid(n_tokens, (C + 255) / 256), sgrid(n_segments, (C + 255) / 256), block(256);
@@ -84,7 +88,8 @@ extern "C" int lmsf_short_conv(const void* u, int dtype, long u_stride, const vo
   // channels, 74 against 60 us, and at 8 tokens, 10.7 against 3.8: its weights' loads lie 64 bytes apart across a wave)
 #define SC(T, A)                                                                                                      \
   hipLaunchKernelGGL((short_conv_kernel<T, A>), grid, block, 0, stream, (const T*)u, u_stride, (const T*)w,           \
-                     (const T*)bias, state, state_stride, seg_of, seg_starts, state_slots, (T*)out, out_stride, C, taps)
+                     (const T*)bias, state, state_stride, seg_of, seg_starts, state_slots, (T*)out, out_stride, C, taps, \
+                     single)
   if (dtype == LMSF_F32) {
     if (act) SC(float, 1); else SC(float, 0);
   } else {
@@ -92,7 +97,7 @@ extern "C" int lmsf_short_conv(const void* u, int dtype, long u_stride, const vo
   }
 #undef SC
   LMSF_LAUNCH_CHECK("short_conv");
-  if (taps > 1) {
+  if (taps > 1 && !single) {
     if (dtype == LMSF_F32)
       hipLaunchKernelGGL((short_conv_state_kernel<float>), sgrid, block, 0, stream, (const float*)u, u_stride, state,
                          state_stride, seg_starts, state_slots, C, taps);

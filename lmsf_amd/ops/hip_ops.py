@@ -803,7 +803,8 @@ class HipOps:
                    batch, activation: Optional[str] = None) -> torch.Tensor:
         """Causal convolution over time, channel by channel: out[t, c] = act(bias[c] + sum_j weight[c, j] u[t - taps + 1 + j, c])
         within each request. ``u`` [N, C] (a view with unit column stride will do), ``weight`` [C, taps]; ``state``
-        float32 [slots, >= C (taps - 1)] holds every request's last taps - 1 inputs and is brought up to date.
+        float32 [slots, >= C (taps - 1)] holds every request's last taps - 1 inputs and is brought up to date (by a
+        second launch, or by the same one in a step of single tokens).
         ``batch`` is the step (engine.batch.StepContext). activation None or "silu"."""
         self._dev(u, weight, bias)
         if u.dim() != 2 or u.stride(1) != 1 or weight.dim() != 2 or weight.shape[0] != u.shape[1] \
@@ -824,7 +825,7 @@ class HipOps:
         self._check(self.lib.lmsf_short_conv(
             _ptr(u), _code(u.dtype), u.stride(0), _ptr(weight), _ptr(bias), 1 if activation else 0, _ptr(state),
             state.stride(0) if state is not None else 0, _ptr(seg_of), _ptr(seg_starts), _ptr(slots), _ptr(out),
-            out.stride(0), N, S, C, taps, self._stream()))
+            out.stride(0), N, S, C, taps, 1 if (getattr(batch, "all_single", False) and S == N) else 0, self._stream()))
         return out
 
     def selective_scan(self, x: torch.Tensor, dt: torch.Tensor, bc: torch.Tensor, b_at: int, c_at: int, z: torch.Tensor,

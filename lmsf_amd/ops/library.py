@@ -10,7 +10,7 @@ from typing import Optional
 from ..csrc import build as _build
 from .dispatch import ProductShape, Route, Tunables
 
-ABI_VERSION = 27
+ABI_VERSION = 28
 
 _lib: Optional[ctypes.CDLL] = None
 _lib_path: Optional[str] = None
@@ -53,7 +53,7 @@ _SIGNATURES = {
     "lmsf_table_moe_grouped": (c_int, [c_int, c_int, c_int, c_int, c_int, c_int, c_long]),
     "lmsf_dyt_norm": (c_int, [_P, c_int, _P, _P, _P, _P, _P, c_int, _P, c_int, c_int, _P]),
     "lmsf_short_conv": (c_int, [_P, c_int, c_long, _P, _P, c_int, _P, c_long, _P, _P, _P, _P, c_long, c_int, c_int, c_int,
-                                c_int, _P]),
+                                c_int, c_int, _P]),
     "lmsf_selective_scan": (c_int, [_P, c_int, c_long, _P, c_long, _P, c_long, c_int, c_int, _P, c_long, _P, _P, _P,
                                     c_long, _P, _P, _P, c_long, c_int, c_int, c_int, c_int, c_int, c_int, _P, _P, _P]),
     "lmsf_selective_scan_entry_floats": (c_long, [c_int, c_int]),

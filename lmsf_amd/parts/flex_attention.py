@@ -65,7 +65,7 @@ class FlexAttention(Mixer):
         bias = [nm["q"], nm["k"], nm["v"]] if qkv_bias else False
         self.proj = FusedLinear(prefix, rt, hidden_size, sources, bias=bias, bare_names=True, bias_name=bias_name)
         self.conv: Optional[ShortConv] = None
-        if conv_taps and int(conv_taps) > 1:
+        if conv_taps and int(conv_taps) >= 1:          # (one tap: a weight per channel, and no state)
             self.conv = ShortConv(prefix, rt, [("%s.%s" % (nm[x], nm["conv"]), n) for x, n in zip("qkv", (
                 H * self.dim, G * self.dim, G * self.vdim))], int(conv_taps))
         self.o = Linear(prefix, rt, nm["o"], H * self.vdim, hidden_size, bare_names=True)
@@ -78,7 +78,9 @@ class FlexAttention(Mixer):
         return CacheSpec(num_kv_heads=self.G, head_dim=self.D, window=self.window)
 
     def state_spec(self) -> Optional[StateSpec]:
-        return StateSpec((self.conv.state_floats,), torch.float32) if self.conv is not None else None
+        if self.conv is None or self.conv.state_floats == 0:
+            return None
+        return StateSpec((self.conv.state_floats,), torch.float32)
 
     def forward(self, h: torch.Tensor, ctx, binding: CacheBinding) -> torch.Tensor:
         ops = self.rt.ops

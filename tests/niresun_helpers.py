@@ -41,7 +41,7 @@ def dense(ff):
 SCALING = {"factor": 8.0, "low": 1.0, "high": 4.0, "original": 64}
 
 # Sizes differ between the configurations and from one another inside each: values wider and narrower than keys,
-# one to six heads, kv heads equal to the heads and fewer, two to five taps, states of 4 to 40 entries (more than 16 a
+# one to six heads, kv heads equal to the heads and fewer, one to five taps, states of 4 to 40 entries (more than 16 a
 # lane group, and not a power of two), chunks that are no multiple of a page, layers in several orders, with and
 # without a feed-forward, rotation over a whole head and over part of it, with and without frequency scaling.
 CONFIGS = {
@@ -61,6 +61,8 @@ CONFIGS = {
     "C": {"architecture": "Niresun", "vocab": 40, "width": 32, "norm": {"eps": 1e-5}, "layers": [
         attn(1, 1, 48, 64, 33, 16, scaling={"factor": 2.0, "low": 2.0, "high": 8.0, "original": 32}),
         mamba(32, 4, 1, 3, mlp=dense(32)),
+        pair(2, 1, 16, 8, 1, (0.25, 1), 2, 8, 8, 2.0),          # filters of one tap: no state of the convolution
+        mamba(24, 20, 2, 1),
     ]},
     # sizes at which the matrix-core attention kernels and the wider state tiles run (GPU tests)
     "M": {"architecture": "Niresun", "vocab": 300, "width": 256, "norm": {"eps": 1e-5}, "layers": [

@@ -250,7 +250,8 @@ def tokens(n, vocab, seed):
     return [rng.randrange(vocab) for _ in range(n)]
 
 
-LAYERS_ALONE = [("A", 0), ("A", 1), ("A", 2), ("B", 0), ("B", 1), ("B", 2), ("B", 3), ("B", 4), ("C", 0), ("M", 2), ("M", 3)]
+LAYERS_ALONE = [("A", 0), ("A", 1), ("A", 2), ("B", 0), ("B", 1), ("B", 2), ("B", 3), ("B", 4), ("C", 0), ("C", 2), ("C", 3),
+                ("M", 2), ("M", 3)]
 
 
 @pytest.mark.parametrize("dtype", ["float32", "bfloat16"])

@@ -162,3 +162,21 @@ def single_layer(which, index, vocab=53):
     cfg = CONFIGS[which]
     return {"architecture": "Niresun", "vocab": vocab, "width": cfg["width"], "norm": cfg["norm"],
             "layers": [cfg["layers"][index]]}
+
+
+def bfloat16_limits(cfg, weights, tokens, ref):
+    """What rounding to bfloat16 may cost at every position: three times what it costs the plain implementation when
+    it rounds what an engine may keep in 16 bits (plain_niresun.storage), but no less than three times the median
+    of that over the positions."""
+    with P.storage(torch.bfloat16):
+        e = row_errs(plain_logits(cfg, weights, tokens), ref)
+    return 3.0 * torch.maximum(e, e.median())
+
+
+def within(got, ref, limits):
+    """Whether ``got`` differs from ``ref`` by rounding only: at most 4 % of the positions (or one) over their limit,
+    none over three times its limit. (One sample of rounding per position is a rough measure, hence the allowance.)
+    Returns (verdict, the worst ratio)."""
+    ratio = row_errs(got, ref) / limits
+    over = int((ratio > 1.0).sum())
+    return bool(over <= max(1, 0.04 * ratio.numel()) and (ratio <= 3.0).all()), float(ratio.max())

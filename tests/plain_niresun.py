@@ -3,15 +3,45 @@
 Written from the design's equations only; it shares nothing with the package. A model is (config dict, dict
 of tensors by checkpoint name). Everything runs in the dtype of the tensors handed in (the tests use float64
 or float32), token by token where the mechanism is a recurrence.
+
+``with storage(torch.bfloat16):`` makes it round what an engine may keep in 16 bits (the operands and results of the
+projections, the convolutions and activations behind them, queries, keys and values, what a mixer or feed-forward
+hands back) while everything else stays as exact as the tensors' dtype: what rounding alone costs, for the tests'
+limits.
 """
+import contextlib
 import math
 
 import torch
 
+_STORAGE = [None]
+
+
+@contextlib.contextmanager
+def storage(dtype):
+    _STORAGE[0] = dtype
+    try:
+        yield
+    finally:
+        _STORAGE[0] = None
+
+
+def kept(x):
+    """x as a 16-bit engine would hold it between two operations."""
+    return x if _STORAGE[0] is None else x.to(_STORAGE[0]).to(x.dtype)
+
+
+def lin(h, w, b=None, wide=False):
+    """h w^T (+ b); ``wide``: the result stays in 32 bits (it enters a recurrence, or is the logits)."""
+    y = kept(h) @ w.T
+    if b is not None:
+        y = y + b
+    return y if wide else kept(y)
+
 
 def dyt(x, w, b, alpha):
     """tanh(alpha x) w + b."""
-    return torch.tanh(alpha * x) * w + b
+    return kept(torch.tanh(alpha * x) * w + b)
 
 
 def unit_rms(x, eps):
@@ -87,11 +117,11 @@ def masked_softmax_attention(q, k, v, scale, visible):
 def mamba1(h, W, p, m):
     """Selective scan. h [T, width]; W name -> tensor; p the layer's prefix with '.mix'."""
     inner, state, rank = m["inner"], m["state"], m["dt_rank"]
-    xz = h @ W[p + ".in"].T
+    xz = lin(h, W[p + ".in"])
     x, z = xz[:, :inner], xz[:, inner:]
-    x = silu(causal_conv(x, W[p + ".conv"], W[p + ".conv.b"]))
-    low = x @ W[p + ".x"].T
-    dt = softplus(low[:, :rank] @ W[p + ".dt"].T + W[p + ".dt.b"])
+    x = kept(silu(causal_conv(x, W[p + ".conv"], W[p + ".conv.b"])))
+    low = lin(x, W[p + ".x"])
+    dt = softplus(lin(low[:, :rank], W[p + ".dt"], W[p + ".dt.b"], wide=True))
     B, C = low[:, rank:rank + state], low[:, rank + state:rank + 2 * state]
     A = -torch.exp(W[p + ".A_log"])
     S = torch.zeros(inner, state, dtype=h.dtype)
@@ -99,53 +129,53 @@ def mamba1(h, W, p, m):
     for t in range(h.shape[0]):
         S = torch.exp(dt[t][:, None] * A) * S + (dt[t] * x[t])[:, None] * B[t][None, :]
         ys.append(S @ C[t] + W[p + ".D"] * x[t])
-    y = torch.stack(ys) * silu(z)
-    return y @ W[p + ".o"].T
+    y = kept(torch.stack(ys) * silu(z))
+    return lin(y, W[p + ".o"])
 
 
 def attention(h, W, p, m, eps):
     """Rotary, chunked, gated softmax attention with biases."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = (h @ W[p + ".q"].T + W[p + ".q.b"]).view(T, H, d)
-    k = (h @ W[p + ".k"].T + W[p + ".k.b"]).view(T, G, d)
-    v = (h @ W[p + ".v"].T + W[p + ".v.b"]).view(T, G, dv)
+    q = lin(h, W[p + ".q"], W[p + ".q.b"]).view(T, H, d)
+    k = lin(h, W[p + ".k"], W[p + ".k.b"]).view(T, G, d)
+    v = lin(h, W[p + ".v"], W[p + ".v.b"]).view(T, G, dv)
     pos = torch.arange(T)
     rot = m.get("rot")               # (a configuration may leave the rotation or the chunks out)
     if rot:
-        q = rotate(q, pos, rot["dims"], rot["base"], rot.get("scaling"))
-        k = rotate(k, pos, rot["dims"], rot["base"], rot.get("scaling"))
+        q = kept(rotate(q, pos, rot["dims"], rot["base"], rot.get("scaling")))
+        k = kept(rotate(k, pos, rot["dims"], rot["base"], rot.get("scaling")))
     size = m["mask"]["size"] if m.get("mask") else 1 << 30
-    o = masked_softmax_attention(q, k, v, m["scale"], lambda i, j: j <= i and i // size == j // size)
-    o = o.reshape(T, H * dv) * torch.sigmoid(h @ W[p + ".g"].T)
-    return o @ W[p + ".o"].T
+    o = kept(masked_softmax_attention(q, k, v, m["scale"], lambda i, j: j <= i and i // size == j // size))
+    o = kept(o.reshape(T, H * dv) * torch.sigmoid(lin(h, W[p + ".g"])))
+    return lin(o, W[p + ".o"])
 
 
 def conv_attention(h, W, p, m, eps):
     """The left half of a parallel mixer: short convolutions, unit-norm q and k, query temperature, causal."""
     T = h.shape[0]
     H, G, d, dv = m["heads"], m["kv_heads"], m["dim"], m["vdim"]
-    q = causal_conv(h @ W[p + ".q"].T, W[p + ".q.conv"]).view(T, H, d)
-    k = causal_conv(h @ W[p + ".k"].T, W[p + ".k.conv"]).view(T, G, d)
-    v = causal_conv(h @ W[p + ".v"].T, W[p + ".v.conv"]).view(T, G, dv)
-    q, k = unit_rms(q, eps), unit_rms(k, eps)
+    q = kept(causal_conv(lin(h, W[p + ".q"]), W[p + ".q.conv"])).view(T, H, d)
+    k = kept(causal_conv(lin(h, W[p + ".k"]), W[p + ".k.conv"])).view(T, G, d)
+    v = kept(causal_conv(lin(h, W[p + ".v"]), W[p + ".v.conv"])).view(T, G, dv)
+    q, k = unit_rms(q, eps), kept(unit_rms(k, eps))
     pos = torch.arange(T)
     if m.get("q_temp"):              # (a configuration may leave the temperature out)
         temp = 1.0 + m["q_temp"]["coef"] * torch.log(torch.floor((pos + 1) / m["q_temp"]["every"]).to(h.dtype) + 1.0)
         q = q * temp[:, None, None]
-    o = masked_softmax_attention(q, k, v, m["scale"], lambda i, j: j <= i)
-    return o.reshape(T, H * dv) @ W[p + ".o"].T
+    o = kept(masked_softmax_attention(kept(q), k, v, m["scale"], lambda i, j: j <= i))
+    return lin(o.reshape(T, H * dv), W[p + ".o"])
 
 
 def mlstm(h, W, p, m, eps):
     """The right half: a matrix memory per head with capped log gates and a running maximum that starts at 0."""
     T = h.shape[0]
     H, d, dv, cap = m["heads"], m["dim"], m["vdim"], m["gate_cap"]
-    q = (h @ W[p + ".q"].T).view(T, H, d) * d ** -0.5
-    k = (h @ W[p + ".k"].T).view(T, H, d)
-    v = (h @ W[p + ".v"].T).view(T, H, dv)
-    gi = cap * torch.tanh((h @ W[p + ".i"].T + W[p + ".i.b"]) / cap)
-    gf = torch.nn.functional.logsigmoid(cap * torch.tanh((h @ W[p + ".f"].T + W[p + ".f.b"]) / cap))
+    q = lin(h, W[p + ".q"]).view(T, H, d) * d ** -0.5
+    k = lin(h, W[p + ".k"]).view(T, H, d)
+    v = lin(h, W[p + ".v"]).view(T, H, dv)
+    gi = cap * torch.tanh(lin(h, W[p + ".i"], W[p + ".i.b"], wide=True) / cap)
+    gf = torch.nn.functional.logsigmoid(cap * torch.tanh(lin(h, W[p + ".f"], W[p + ".f.b"], wide=True) / cap))
     S = torch.zeros(H, d, dv, dtype=h.dtype)
     n = torch.zeros(H, d, dtype=h.dtype)
     mx = torch.zeros(H, dtype=h.dtype)
@@ -160,18 +190,18 @@ def mlstm(h, W, p, m, eps):
         den = torch.maximum((n * q[t]).sum(-1).abs(), torch.exp(-mx)) + 1e-6
         outs.append(num / den[:, None])
     o = unit_rms(torch.stack(outs), eps).reshape(T, H * dv) * W[p + ".norm"]
-    o = o * torch.sigmoid(h @ W[p + ".g"].T)
-    return o @ W[p + ".o"].T
+    o = kept(o * torch.sigmoid(lin(h, W[p + ".g"])))
+    return lin(o, W[p + ".o"])
 
 
 def parallel(h, W, p, m, eps):
     a = unit_rms(conv_attention(h, W, p + ".left", m["left"], eps), eps) * W[p + ".left.out"]
     b = unit_rms(mlstm(h, W, p + ".right", m["right"], eps), eps) * W[p + ".right.out"]
-    return 0.5 * (a + b)
+    return kept(0.5 * (a + b))
 
 
 def dense_ffn(h, W, p):
-    return (gelu_tanh(h @ W[p + ".gate"].T) * (h @ W[p + ".up"].T)) @ W[p + ".down"].T
+    return lin(kept(gelu_tanh(lin(h, W[p + ".gate"])) * lin(h, W[p + ".up"])), W[p + ".down"])
 
 
 MIXERS = {"mamba1": lambda h, W, p, m, eps: mamba1(h, W, p, m), "attention": attention, "parallel": parallel}
@@ -190,5 +220,5 @@ def forward(config, W, tokens, want_layers=False):
             h = dyt(x, W[p + ".norm2"], W[p + ".norm2.b"], W[p + ".norm2.alpha"])
             x = x + dense_ffn(h, W, p + ".mlp")
         after.append(x)
-    logits = dyt(x, W["final.norm"], W["final.norm.b"], W["final.norm.alpha"]) @ W["head"].T
+    logits = lin(dyt(x, W["final.norm"], W["final.norm.b"], W["final.norm.alpha"]), W["head"], wide=True)
     return (logits, torch.stack(after)) if want_layers else logits

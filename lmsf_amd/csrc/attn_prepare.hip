@@ -96,7 +96,9 @@ extern "C" int lmsf_attn_prepare(const void* q, long q_stride, const void* k, lo
   LMSF_CHECK(!slots || (k_pages && v_pages && ps > 0 && num_pages > 0), "attn_prepare: slots without pages");
   LMSF_CHECK(temp_every >= 0, "attn_prepare: negative temperature period");
   if (n_tokens == 0) return 0;
-  const dim3 grid(n_tokens, std::min((H + 2 * G + 3) / 4, 65535));
+  // few tokens: the heads spread over workgroups (8 tokens: 8.4 -> 4.1 us); many: a workgroup a token walks its heads
+  // (2,048 tokens: 17.4 us against 23 with the heads spread)
+  const dim3 grid(n_tokens, n_tokens >= 256 ? 1 : std::min((H + 2 * G + 3) / 4, 65535));
   if (dtype == LMSF_F32)
     hipLaunchKernelGGL((attn_prepare_kernel<float>), grid, dim3(256), 0, stream, (const float*)q, q_stride,
                        (const float*)k, k_stride, (const float*)v, v_stride, positions, table, rot, max_pos, slots,

@@ -1117,6 +1117,30 @@ class HipOps:
                                                  _code(out_dtype), y.stride(0), M, N, K, self._stream()))
         return y
 
+    def linear_wide(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None) -> torch.Tensor:
+        """x weight^T + bias in float32, for results that enter a recurrence (a step size, a gate). With many
+        bfloat16 rows the product runs in the many-rows matrix-core kernel with K in two parts, whose float32 partial
+        sums the reduction kernel adds up with the bias (the BLAS library's plans of this package write bfloat16
+        only, and ``linear`` would cut the rows into pieces of ``mid_max_rows``: 16 launches for 2,048 rows);
+        otherwise it is ``linear`` with float32 output."""
+        M, K = x.shape
+        N = weight.shape[0]
+        if (x.dtype == torch.bfloat16 and weight.dtype == torch.bfloat16 and M > self.mid_max_rows and x.dim() == 2
+                and weight.dim() == 2 and weight.shape[1] == K and K % 64 == 0 and K >= 128 and N % 8 == 0
+                and x.stride(1) == 1 and weight.stride(1) == 1 and x.stride(0) % 8 == 0 and weight.stride(0) % 8 == 0
+                and x.data_ptr() % 16 == 0 and weight.data_ptr() % 16 == 0
+                and (bias is None or (bias.shape == (N,) and bias.dtype == weight.dtype and bias.is_contiguous()))):
+            self._dev(x, weight, bias)
+            plan = self.lib.lmsf_gemm_large_plan(M, N, K, 0) // 16 * 16 + 2
+            parts = torch.empty((2, M, N), dtype=torch.float32, device=x.device)
+            self._check(self.lib.lmsf_gemm_large(_ptr(x), x.stride(0), _ptr(weight), weight.stride(0), None, None, 0,
+                                                 M, N, K, 0, plan, _ptr(parts), 0, self._stream()))
+            y = torch.empty((M, N), dtype=torch.float32, device=x.device)
+            self._check(self.lib.lmsf_gemm_mid_reduce(_ptr(parts), _ptr(bias), _ptr(y), F32, y.stride(0), M, N, 2,
+                                                      self._stream()))
+            return y
+        return self.linear(x, weight, bias, out_dtype=torch.float32)
+
     def linear_gated(self, x: torch.Tensor, weight: torch.Tensor, bias: Optional[torch.Tensor] = None,
                      kind: str = "silu") -> torch.Tensor:
         """act(x Wg^T + bg) * (x Wu^T + bu) for the fused weight [2 I, K] = [Wg; Wu] (bias [2 I] likewise);

@@ -114,7 +114,7 @@ class SelectiveScan(Mixer):
         xz = self.in_proj.forward(h)                                            # [N, 2 inner]
         x = self.conv.forward(xz[:, :self.inner], ctx, st[:, self.scan_floats:] if self.taps > 1 else None)
         low = self.x_proj.forward(x)                                            # [N, rank + 2 n]: dt, B, C
-        dt = ops.linear(low[:, :self.rank], self.dt_proj.weight, self.dt_proj.bias, out_dtype=torch.float32)
+        dt = ops.linear_wide(low[:, :self.rank], self.dt_proj.weight, self.dt_proj.bias)   # float32: a step size
         y = ops.selective_scan(x, dt, low, self.rank, self.rank + self.n, xz[:, self.inner:], self.a_log.weight,
                                self.d.weight, st, ctx)
         return self.o.forward(y)
@@ -160,7 +160,7 @@ class MatrixMemory(Mixer):
         ops = self.rt.ops
         H, d, dv = self.H, self.d, self.dv
         p = self.qkvg.forward(h)
-        gates = ops.linear(h, self.gates.weight, self.gates.bias, out_dtype=torch.float32)      # [N, 2 H]
+        gates = ops.linear_wide(h, self.gates.weight, self.gates.bias)                         # float32 [N, 2 H]
         o = ops.mlstm(p[:, :H * d], p[:, H * d:2 * H * d], p[:, 2 * H * d:2 * H * d + H * dv], gates,
                       p[:, 2 * H * d + H * dv:], self.norm.weight, binding.state, ctx, H, d, dv, d ** -0.5, self.cap,
                       self.eps)

@@ -380,6 +380,9 @@ class TorchOps:
         y = y.to(out_dtype or x.dtype)
         return y if out is None else out.copy_(y)
 
+    def linear_wide(self, x, weight, bias=None):
+        return self.linear(x, weight, bias, out_dtype=torch.float32)
+
     def materialize(self, y):
         return y
 

@@ -7,6 +7,7 @@
 // head size (core/src/model_executor/layers/attention.rs:91-103) and rotates and stores in two kernels
 // (vllm/kernels/pos_encoding_kernels.cu:12-36, cache_kernels.cu:150-214).
 #include "common.h"
+#include "entry_points.h"
 
 #include <math.h>
 

@@ -9,6 +9,7 @@
 // float32; branch and out are float32 or bfloat16. The reference's only norm is RMSNorm
 // (vllm/kernels/layernorm_kernels.cu:13-38), with the same fused addition (:41-68).
 #include "common.h"
+#include "entry_points.h"
 
 #include <math.h>
 

@@ -50,6 +50,44 @@ int lmsf_table_moe(const void* h, int dtype, long h_stride, const void* Wgu, con
 long lmsf_table_moe_scratch_ints(int n_tokens, int top, int E);
 int lmsf_table_moe_grouped(int dtype, int n_tokens, int top, int E, int F, int W, long h_stride);
 
+// attn_prepare.hip
+int lmsf_attn_prepare(const void* q, long q_stride, const void* k, long k_stride, const void* v, long v_stride, int
+    dtype, const int* positions, const float* table, int rot, int max_pos, const int* slots, void* q_out, long
+    qo_stride, void* k_pages, void* v_pages, long num_pages, int n_tokens, int H, int G, int dim, int vdim, int D, int
+    ps, int unit_norm, float eps, float temp_coef, int temp_every, hipStream_t stream);
+int lmsf_head_gate(const void* x, int dtype, long x_stride, int x_head, const void* gate, long gate_stride, void* out,
+    long out_stride, int n_tokens, int H, int dv, hipStream_t stream);
+int lmsf_rms_pair(const void* a, long a_stride, const void* b, long b_stride, int dtype, const float* wa, const float*
+    wb, void* out, int n_rows, int W, float eps, float scale, hipStream_t stream);
+
+// dyt_norm.hip
+int lmsf_dyt_norm(const void* branch, int branch_dtype, float* residual, const float* w, const float* b, const float*
+    alpha, void* out, int out_dtype, const int* rows, int n_rows, int H, hipStream_t stream);
+
+// recurrent.hip
+int lmsf_short_conv(const void* u, int dtype, long u_stride, const void* w, const void* bias, int act, float* state,
+    long state_stride, const int* seg_of, const int* seg_starts, const int* state_slots, void* out, long out_stride,
+    int n_tokens, int n_segments, int C, int taps, int single, hipStream_t stream);
+long lmsf_selective_scan_entry_floats(int inner, int nstate);
+int lmsf_selective_scan(const void* x, int dtype, long x_stride, const float* dt_pre, long dt_stride, const void* bc,
+    long bc_stride, int b_at, int c_at, const void* z, long z_stride, const float* A_log, const float* Dw, float*
+    state, long state_stride, const int* seg_starts, const int* state_slots, void* y, long y_stride, int n_tokens, int
+    n_segments, int inner, int nstate, int chunk, int max_chunks, const int* scratch_base, float* scratch,
+    hipStream_t stream);
+long lmsf_mlstm_state_floats(int H, int d, int dv);
+long lmsf_mlstm_chunk_scratch_floats(int n_tokens, int H, int dv);
+int lmsf_mlstm_chunk_tokens(int d);
+long lmsf_mlstm_chunk_entry_floats(int H, int d, int dv);
+int lmsf_mlstm_chunked(const void* q, const void* k, const void* v, int dtype, long qkv_stride, const float* gates,
+    long gates_stride, const void* og, long og_stride, const float* norm_w, float* state, long state_stride, const
+    int* seg_starts, const int* state_slots, void* out, long out_stride, float* o_raw, int n_tokens, int n_segments,
+    int H, int d, int dv, float qscale, float cap, float eps, const int* chunk_base, int max_chunks, long n_entries,
+    float* entries, hipStream_t stream);
+int lmsf_mlstm_tokens(const void* q, const void* k, const void* v, int dtype, long qkv_stride, const float* gates,
+    long gates_stride, const void* og, long og_stride, const float* norm_w, float* state, long state_stride, const
+    int* seg_starts, const int* state_slots, void* out, long out_stride, float* o_raw, int n_tokens, int n_segments,
+    int H, int d, int dv, float qscale, float cap, float eps, hipStream_t stream);
+
 // blas.hip
 int lmsf_blas_init(long workspace_bytes);
 int lmsf_blas_ready();

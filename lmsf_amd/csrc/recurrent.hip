@@ -11,6 +11,7 @@
 // (portions of prompts) take forms that work on chunks of tokens at once; they and the token-by-token forms agree up
 // to rounding. All arithmetic is float32.
 #include "common.h"
+#include "entry_points.h"
 
 #include <math.h>
 

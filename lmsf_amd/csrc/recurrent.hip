@@ -452,12 +452,18 @@ extern "C" int lmsf_selective_scan(const void* x, int dtype, long x_stride, cons
 //   o = S^T q / (max(|n . q|, exp(-m')) + 1e-6),  q times qscale;
 //   out = o / rms(o) * w * sigmoid(g)      (rms over the head's dv entries, eps inside the root)
 // n is kept as one more column of S (a value entry that is always 1), so that n . q comes out of the same sums as
-// S^T q. The state of a slot: S and n as [H, d, dv + 1], then m as [H].
+// S^T q. The state of a slot: S and n as [H, d, dv + 1], then m as [H, copies] (below).
 // Three forms follow: chunks of a segment one after the other or side by side (portions of prompts), and token by
 // token with the memory streamed once (steps of single tokens).
 
-// floats of state a slot needs: S and n as [H, d, dv + 1], m as [H]
-extern "C" long lmsf_mlstm_state_floats(int H, int d, int dv) { return (long)H * d * (dv + 1) + H; }
+// floats of state a slot needs
+// m is kept once per block of 32 value columns (all copies equal): workgroups that take different blocks of one head
+// then share nothing that any of them writes, whichever of them starts first.
+#define MLS_M_COLS 32
+__host__ __device__ static inline int mls_m_copies(int dv) { return (dv + MLS_M_COLS - 1) / MLS_M_COLS; }
+extern "C" long lmsf_mlstm_state_floats(int H, int d, int dv) {
+  return (long)H * d * (dv + 1) + (long)H * mls_m_copies(dv);
+}
 
 // ---------------------------------------------------------------- the matrix memory over chunks of tokens
 // The same recurrence for segments of many tokens, a chunk of L tokens at a time. With F_t the sum of the log forget
@@ -512,7 +518,7 @@ __global__ __launch_bounds__(MLC_THREADS) void mlstm_chunk_kernel(
   float* st = state + (long)state_slots[s] * state_stride;
   // where S_0 comes from (and, MODE 0, goes back to) and where m_0 lies
   float* gS = MODE == 0 ? st + (long)h * d * cols : sc_U + (ent * H + h) * d * cols;
-  float* gm = MODE == 0 ? st + (long)H * d * cols + h : sc_m0 + ent * H + h;
+  float* gm = MODE == 0 ? st + (long)H * d * cols + (long)h * mls_m_copies(dv) + vb : sc_m0 + ent * H + h;
   if (MODE != 1) {
     for (int i = tid; i < d * NC; i += MLC_THREADS) {
       const int dd = i / NC, c = i % NC;
@@ -611,7 +617,8 @@ __global__ __launch_bounds__(MLC_THREADS) void mlstm_chunk_kernel(
       }
       m = sF[nt - 1] + M_last;
     }
-    if (MODE == 2 && end == seg_end && vb == 0 && tid == 0) st[(long)H * d * cols + h] = sF[nt - 1] + M_last;
+    if (MODE == 2 && end == seg_end && tid == 0)
+      st[(long)H * d * cols + (long)h * mls_m_copies(dv) + vb] = sF[nt - 1] + M_last;      // this block's copy of m
     if (MODE == 1) {
       // U = K^T (w [V | 1]) straight to the scratch; (F_last, G) beside it
       for (int i = tid; i < d * NC; i += MLC_THREADS) {
@@ -635,7 +642,7 @@ __global__ __launch_bounds__(MLC_THREADS) void mlstm_chunk_kernel(
       if (c < nb) gS[(long)dd * cols + e0 + c] = sS[dd * NCp + c];
       else if (vb == 0) gS[(long)dd * cols + dv] = sS[dd * NCp + c];
     }
-    if (tid == 0 && vb == 0) gm[0] = m;
+    if (tid == 0) gm[0] = m;                     // this block's copy
   }
 }
 
@@ -655,7 +662,7 @@ __global__ __launch_bounds__(256) void mlstm_fold_kernel(float* __restrict__ sta
   const int n_chunks = (seg_starts[s + 1] - seg_starts[s] + L - 1) / L;
   float* st = state + (long)state_slots[s] * state_stride;
   float S = st[(long)h * per + i];
-  float m = st[(long)H * per + h];
+  float m = st[(long)H * per + (long)h * mls_m_copies(dv)];      // (copy 0; nobody writes m in this launch)
   const long base = chunk_base[s];
   for (int j = 0; j < n_chunks; ++j) {
     const long ent = (base + j) * H + h;
@@ -716,7 +723,7 @@ __global__ __launch_bounds__(256) void mlstm_token_kernel(
   const bool col_ok = e0 + lane < dv;
   float* st = state + (long)state_slots[s] * state_stride;
   float* gS = st + (long)h * d * cols;
-  float* gm = st + (long)H * d * cols + h;
+  float* gm = st + (long)H * d * cols + (long)h * mls_m_copies(dv) + blockIdx.z * (MLD_COLS / MLS_M_COLS);
   float m = gm[0];
   for (int t = seg_starts[s]; t < seg_starts[s + 1]; ++t) {
     __syncthreads();
@@ -766,7 +773,7 @@ __global__ __launch_bounds__(256) void mlstm_token_kernel(
       o_raw[(long)t * o_stride + h * dv + e0 + lane] =
           so[lane] + so[MLD_COLS + lane] + so[2 * MLD_COLS + lane] + so[3 * MLD_COLS + lane];
   }
-  if (tid == 0 && blockIdx.z == 0) gm[0] = m;
+  if (tid < MLD_COLS / MLS_M_COLS && e0 + tid * MLS_M_COLS < dv) gm[tid] = m;       // this block's copies of m
 }
 
 // the temporary of the forms that leave the division to the heads' kernel: numerators float32 [n_tokens, H * dv], then
@@ -808,7 +815,7 @@ extern "C" int lmsf_mlstm_chunked(const void* q, const void* k, const void* v, i
   LMSF_CHECK(n_tokens >= 0 && n_segments >= 0 && n_segments <= 65535, "mlstm_chunked: bad counts");
   LMSF_CHECK(!chunk_base || (entries && max_chunks >= 1 && n_entries >= 1), "mlstm_chunked: chunks without scratch");
   if (n_tokens == 0 || n_segments == 0) return 0;
-  const int DVB = 32, NCp = (DVB + 1) | 1, dp = d | 1;
+  const int DVB = MLS_M_COLS, NCp = (DVB + 1) | 1, dp = d | 1;       // (a block of columns owns one copy of m)
   const int L = lmsf_mlstm_chunk_tokens(d);
   LMSF_CHECK(L > 0, "mlstm_chunked: heads of %d entries do not fit a workgroup's LDS", d);
   const size_t smem = ((size_t)2 * L * dp + (size_t)2 * L * NCp + (size_t)L * (L | 1) + (size_t)d * NCp + 4 * L) * sizeof(float);

@@ -146,6 +146,15 @@ __device__ __forceinline__ void rope_rotate(float x, float y, float c, float s, 
   *yr = __fmaf_rn(y, c, __fmul_rn(x, s));
 }
 
+// The activation of a gated product by its code: 1 SiLU, 2 GELU in the erf form, 5 GELU in the tanh form
+// x/2 (1 + tanh(sqrt(2/pi) (x + 0.044715 x^3))) (3 and 4 are forms of the products that are no activations).
+template <int ACT>
+__device__ __forceinline__ float gated_product_activation(float g) {
+  if (ACT == 1) return g / (1.0f + expf(-g));
+  if (ACT == 2) return 0.5f * g * (1.0f + erff(g * 0.70710678118654752f));
+  return 0.5f * g * (1.0f + tanhf(0.79788456080286536f * (g + 0.044715f * g * g * g)));
+}
+
 // The first key position that a query at position p attends to; the last is p itself. ``window`` > 0: the last
 // ``window`` positions; < 0: the positions of p's own chunk of -window positions, chunks counted from position 0 of
 // the request (wherever a prompt was cut into steps); 0: every position. It never falls as p rises.

@@ -71,7 +71,7 @@ struct NormAroundArgs {
   int H;                      // columns of the stream: the mean is over these
 };
 
-// ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated, 3 rotary embedding and cache write,
+// ACT: 0 none (plain linear layer), 1 silu-gated, 2 gelu-gated (5: its tanh form), 3 rotary embedding and cache write,
 // 4 add to the stream and prepare the norm that follows (y receives bf16(stream * w))
 // XROWS: rows of a tile of x that are fetched and staged, 16 or (one row tile of up to 8 rows) 8; the columns of the
 // result that belong to the others are never stored.
@@ -82,7 +82,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
                                                               long ldy, int M, int N, int K, RopeCacheArgs rc,
                                                               NormAroundArgs na) {
   using T = SkinnyTile<KC>;
-  constexpr int WT = (ACT >= 1 && ACT <= 3) ? 2 : 1;   // W tiles per chunk: gate and up, the two halves of a head, or one
+  constexpr int WT = ((ACT >= 1 && ACT <= 3) || ACT == 5) ? 2 : 1;   // W tiles per chunk: gate and up, the two halves of a head, or one
   constexpr int XLOADS = (XROWS + T::ROWS_PER_LOAD - 1) / T::ROWS_PER_LOAD;   // load instructions per tile of x
   static_assert(XROWS == 16 || (XROWS == 8 && MT == 1 && XLOADS < T::LOADS), "8 rows of x: one row tile, and a whole load fewer");
   static_assert(!(SCALED || ACT == 4) || MT == 1, "the forms around a norm take up to 16 rows");
@@ -325,8 +325,7 @@ __global__ __launch_bounds__(NW * 64) void gemm_skinny_kernel(const bf16_t* __re
         // stores them (so both paths give the same bits)
         g = bf16_to_f32(f32_to_bf16(g));
         u = bf16_to_f32(f32_to_bf16(u));
-        const float a = ACT == 1 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + erff(g * 0.70710678118654752f));
-        r = a * u;
+        r = gated_product_activation<ACT>(g) * u;
       }
       y[(long)m * ldy + n] = from_f32<TOut>(r);
     }
@@ -349,7 +348,7 @@ template <int MT, int KC, int NW, typename TOut, int ACT, int DEPTH, bool SCALED
 static int launch_skinny_x(const void* x, long ldx, const void* W, long ldw, const void* bias, void* y, long ldy, int M,
                            int N, int K, hipStream_t stream, RopeCacheArgs rc, NormAroundArgs na) {
   using T = SkinnyTile<KC>;
-  constexpr int WT = (ACT >= 1 && ACT <= 3) ? 2 : 1;
+  constexpr int WT = ((ACT >= 1 && ACT <= 3) || ACT == 5) ? 2 : 1;
   const size_t stage = (size_t)NW * (WT + MT) * T::TILE_BYTES;
   const size_t red = (size_t)NW * WT * MT * 64 * 4 * sizeof(float) + ((SCALED || ACT == 4) ? 256 * sizeof(float) : 0);
   const size_t smem = stage > red ? stage : red;
@@ -398,22 +397,24 @@ extern "C" int lmsf_gemm_skinny(const void* x, long ldx, const void* W, long ldw
              "gemm_skinny: row strides must cover K and be multiples of 8");
   LMSF_CHECK(lmsf_aligned16(x) && lmsf_aligned16(W), "gemm_skinny: x and W must be 16-byte aligned");
   LMSF_CHECK(out_dtype == LMSF_F32 || out_dtype == LMSF_BF16, "gemm_skinny: unknown output dtype %d", out_dtype);
-  LMSF_CHECK(act >= 0 && act <= 2, "gemm_skinny: unknown activation %d", act);
+  LMSF_CHECK((act >= 0 && act <= 2) || act == 5, "gemm_skinny: unknown activation %d", act);
   LMSF_CHECK(act == 0 || out_dtype == LMSF_BF16, "gemm_skinny: the gated form writes bfloat16 only");
   if (M == 0) return 0;
   const int mt = (M + 15) / 16;
   int rc = 0;
   if (act) {
 #define SKG(MT_, KC_, NW_)                                                                                     \
-  rc = act == 1 ? launch_skinny<MT_, KC_, NW_, bf16_t, 1>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)       \
-                : launch_skinny<MT_, KC_, NW_, bf16_t, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
+  rc = act == 1   ? launch_skinny<MT_, KC_, NW_, bf16_t, 1>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)     \
+       : act == 2 ? launch_skinny<MT_, KC_, NW_, bf16_t, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)     \
+                  : launch_skinny<MT_, KC_, NW_, bf16_t, 5>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
     if (mt == 1) {
       // 8 waves with two chunks each in flight: measured 3 % ahead of 16 waves with one (deeper: slower)
       if (variant == 1) SKG(1, 128, 8);
       else if (variant == 3) SKG(1, 64, 16);
       else   // (variant 2 of the plain product splits K over 8 waves as well: the same order of summation)
-        rc = act == 1 ? launch_skinny<1, 64, 8, bf16_t, 1, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
-                      : launch_skinny<1, 64, 8, bf16_t, 2, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream);
+        rc = act == 1   ? launch_skinny<1, 64, 8, bf16_t, 1, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
+             : act == 2 ? launch_skinny<1, 64, 8, bf16_t, 2, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream)
+                        : launch_skinny<1, 64, 8, bf16_t, 5, 2>(x, ldx, W, ldw, bias, y, ldy, M, N, K, stream);
     } else if (mt == 2) {
       SKG(2, 64, 16);
     } else if (mt == 3) {

@@ -17,7 +17,7 @@
 // SC takes that norm's row factor out of the product (see GemvNorm). The addition and the norm are then no
 // kernels of their own (vllm/kernels/layernorm_kernels.cu:41-68 in the reference).
 //
-// A "unit" is what one wave produces: ACT 0: output n (one row of W); ACT 1, 2: output n of the gated form
+// A "unit" is what one wave produces: ACT 0: output n (one row of W); ACT 1, 2, 5: output n of the gated form
 // (rows n and N + n: gate and up); ACT 3: the rotation pair (i, i + d/2) of one head of the fused QKV
 // projection (rows head * d + i and head * d + i + d/2).
 #include "common.h"
@@ -164,11 +164,10 @@ __global__ __launch_bounds__(GEMV_WAVES * 64) void gemv_kernel(const bf16_t* __r
           nm.xw_out[(long)m * nm.ld_xw + n] = f32_to_bf16(v * (bf16_to_f32(nm.weight[n]) + nm.offset));
           sq_acc[m] += v * v;
         }
-      } else if (ACT == 1 || ACT == 2) {
+      } else if (ACT == 1 || ACT == 2 || ACT == 5) {
         // the two products are rounded to the storage type before the activation, as the unfused path stores them
         const float g = bf16_to_f32(f32_to_bf16(a)), u = bf16_to_f32(f32_to_bf16(b));
-        const float act = ACT == 1 ? g / (1.0f + expf(-g)) : 0.5f * g * (1.0f + erff(g * 0.70710678118654752f));
-        y[(long)m * ldy + n] = from_f32<TOut>(act * u);
+        y[(long)m * ldy + n] = from_f32<TOut>(gated_product_activation<ACT>(g) * u);
       } else {
         // rounded to the storage type first, as the product stores them when the rotation is a kernel of its own
         a = bf16_to_f32(f32_to_bf16(a));
@@ -318,7 +317,7 @@ extern "C" int lmsf_gemv(const void* x, long ldx, const void* W, long ldw, const
                          long ldy, int M, int N, int K, int act, hipStream_t stream) {
   if (int rc = gemv_check("gemv", x, ldx, W, ldw, M, N, K)) return rc;
   LMSF_CHECK(y != nullptr && ldy >= N, "gemv: bad output");
-  LMSF_CHECK(act >= 0 && act <= 2, "gemv: unknown activation %d", act);
+  LMSF_CHECK((act >= 0 && act <= 2) || act == 5, "gemv: unknown activation %d", act);
   LMSF_CHECK(out_dtype == LMSF_BF16 || (out_dtype == LMSF_F32 && act == 0),
              "gemv: output is bfloat16, or float32 without activation");
   if (M == 0) return 0;
@@ -326,6 +325,7 @@ extern "C" int lmsf_gemv(const void* x, long ldx, const void* W, long ldw, const
 #define GV(NX_)                                                                                              \
   r = act == 1   ? launch_gemv<NX_, 1, bf16_t>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream)                 \
       : act == 2 ? launch_gemv<NX_, 2, bf16_t>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream)                 \
+      : act == 5 ? launch_gemv<NX_, 5, bf16_t>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream)                 \
       : out_dtype == LMSF_F32 ? launch_gemv<NX_, 0, float>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream)     \
                               : launch_gemv<NX_, 0, bf16_t>(x, ldx, W, ldw, bias, y, ldy, N, K, N, stream)
   if (M == 1) GV(1); else GV(2);

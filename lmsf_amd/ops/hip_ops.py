@@ -1151,10 +1151,7 @@ class HipOps:
         split K over 8 and over 16 waves). ``x`` may be a ``ScaledRows``."""
         if weight.dim() != 2 or weight.shape[0] % 2 != 0:
             raise ValueError("linear_gated: weight must be [2 I, K]")
-        if kind == "gelu_tanh":
-            # (no product has this activation as its epilogue: the product, then the activation kernel)
-            return self.gated_act(self.linear(self.materialize(x), weight, bias), kind)
-        kinds = {"silu": 1, "gelu": 2}
+        kinds = {"silu": 1, "gelu": 2, "gelu_tanh": 5}
         if kind not in kinds:
             raise ValueError("unknown activation %r (known: %s)" % (kind, ", ".join(kinds)))
         M, I = x.shape[0], weight.shape[0] // 2
@@ -1168,8 +1165,9 @@ class HipOps:
                                          x.rows_per_tile if scaled else 0, x.tiles if scaled else 0, ctypes.byref(rt))
         if rt.route == D.MATERIALIZE:
             return self.linear_gated(self.materialize(x), weight, bias, kind)
-        if rt.route == D.SEPARATE:
-            return self.gated_act(self.linear(x, weight, bias), kind)
+        if rt.route == D.SEPARATE or (kind == "gelu_tanh" and rt.route not in (D.GEMV, D.SKINNY)):
+            # (the tanh form of GELU is an epilogue of the one-row and the few-rows product only)
+            return self.gated_act(self.linear(self.materialize(x), weight, bias), kind)
         self._dev(xt, weight, bias)
         if bias is not None and (bias.shape != (2 * I,) or bias.dtype != weight.dtype or not bias.is_contiguous()):
             raise ValueError("linear_gated: bias must be [%d] of the weight's dtype" % (2 * I))

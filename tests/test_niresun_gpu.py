@@ -108,6 +108,19 @@ def test_gated_activation_in_the_tanh_form(dtype):
 
 
 @pytest.mark.parametrize("dtype", DTYPES)
+@pytest.mark.parametrize("rows", [1, 2, 8, 16, 40, 300])
+def test_gated_product_with_the_tanh_form(dtype, rows):
+    """One and few rows: the activation is the product's epilogue; more rows: the product, then the activation kernel."""
+    g = torch.Generator().manual_seed(rows)
+    K, I = 256, 136
+    x = torch.randn((rows, K), generator=g).to(dtype)
+    w = (torch.randn((2 * I, K), generator=g) / 16).to(dtype)
+    got = ops().linear_gated(x.cuda(), w.cuda(), None, "gelu_tanh")
+    gate, up = (x.double() @ w[:I].double().T).to(dtype).double(), (x.double() @ w[I:].double().T).to(dtype).double()
+    close(got, P.gelu_tanh(gate) * up, dtype, scale=2.0)
+
+
+@pytest.mark.parametrize("dtype", DTYPES)
 @pytest.mark.parametrize("C,taps,act,off", [(24, 3, None, 2), (300, 4, "silu", 2), (8, 2, None, 8), (40, 7, "silu", 8),
                                             (16, 1, None, 2), (512, 4, "silu", 8), (72, 3, None, 8)])
 def test_short_convolution_over_cut_requests(dtype, C, taps, act, off):

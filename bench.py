@@ -451,8 +451,8 @@ def niresun_shapes(name):
         "mlp": {"kind": "dense", "ff": ff}}
     par = {"type": "parallel", "mixer": {
         "left": {"heads": H, "kv_heads": max(1, H // 4), "dim": d // 2, "vdim": d // 2, "scale": (d // 2) ** -0.5,
-                 "conv": taps, "q_temp": {"coef": 0.5, "every": 1024}},
-        "right": {"heads": max(1, H // 2), "dim": d, "vdim": d, "gate_cap": 15.0}}, "mlp": {"kind": "dense", "ff": ff}}
+                 "conv": taps, "q_temp": {"coef": 0.3, "every": 1024}},
+        "right": {"heads": max(1, H // 2), "dim": d, "vdim": d, "gate_cap": 20.0}}, "mlp": {"kind": "dense", "ff": ff}}
     layers = [(scan, att, scan, par)[i % 4] for i in range(L)]
     nire = {"architecture": "Niresun", "vocab": V, "width": W, "norm": {"eps": 1e-5}, "layers": layers,
             "max_position_embeddings": 8192, "torch_dtype": "bfloat16"}

@@ -48,7 +48,7 @@ CONFIGS = {
     "A": {"architecture": "Niresun", "vocab": 61, "width": 48, "norm": {"eps": 1e-5}, "layers": [
         mamba(72, 8, 5, 4),
         attn(4, 2, 16, 24, 20, 8, scaling=SCALING, mlp=dense(96)),
-        pair(4, 2, 16, 16, 3, (0.5, 8), 2, 24, 16, 15.0, mlp=dense(64)),
+        pair(4, 2, 16, 16, 3, (0.4, 8), 2, 24, 16, 12.0, mlp=dense(64)),
         mamba(72, 8, 5, 4, mlp=dense(80)),
     ]},
     "B": {"architecture": "Niresun", "vocab": 77, "width": 64, "norm": {"eps": 1e-6}, "layers": [
@@ -68,7 +68,7 @@ CONFIGS = {
     "M": {"architecture": "Niresun", "vocab": 300, "width": 256, "norm": {"eps": 1e-5}, "layers": [
         mamba(512, 16, 16, 4),
         attn(8, 2, 64, 96, 48, 32, scaling=SCALING, mlp=dense(512)),
-        pair(8, 4, 64, 64, 4, (0.5, 16), 4, 64, 128, 15.0, mlp=dense(384)),
+        pair(8, 4, 64, 64, 4, (0.3, 16), 4, 64, 128, 10.0, mlp=dense(384)),
         mamba(512, 72, 16, 4),
     ]},
 }

@@ -32,8 +32,8 @@ def draw_config(seed):
             return attn(heads, kv, dim, pick([8, 12, 24, 40, 80]), pick([None, 5, 16, 37, 64, 130]), rot,
                         base=pick([100.0, 10000.0, 1e6]), scaling=pick([None, SCALING]) if rot else None,
                         scale=pick([None, 0.2]), mlp=mlp())
-        return pair(heads, kv, dim, pick([8, 20, 24, 48]), pick([1, 2, 3, 5]), pick([None, (0.5, 7), (2.0, 64)]),
-                    pick([1, 2, 3]), pick([8, 20, 48]), pick([8, 12, 40, 80]), pick([2.0, 15.0, 50.0]), mlp=mlp())
+        return pair(heads, kv, dim, pick([8, 20, 24, 48]), pick([1, 2, 3, 5]), pick([None, (0.6, 7), (2.0, 50)]),
+                    pick([1, 2, 3]), pick([8, 20, 48]), pick([8, 12, 40, 80]), pick([2.0, 14.0, 50.0]), mlp=mlp())
 
     cfg = {"architecture": "Niresun", "vocab": pick([41, 97, 256, 331]), "width": pick([40, 72, 100, 136, 256]),
            "norm": {"eps": pick([1e-5, 1e-6])}, "layers": [layer() for _ in range(pick([2, 3, 4, 5]))]}
